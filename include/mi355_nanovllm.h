@@ -636,6 +636,77 @@ int mi_comm_status(mi_comm* comm, int* timed_out);
  * the peer is ahead)}.  Synchronous; meaningful once mi_comm_status reports a time-out.  Bring-up aid. */
 int mi_comm_timeout_info(mi_comm* comm, uint32_t info[4]);
 
+/* ---- 32-bit-residual model families: general projections, sequence mixers, grouped routing ----------------
+ * (csrc/gemm_any.hip, csrc/seqmix.hip.)  Activations are fp32 throughout; `*_dtype` arguments name the storage
+ * of weights / tables / K-V caches: */
+#define MI_DTYPE_BF16 0
+#define MI_DTYPE_F32  1
+/* A step's rows: cu_q [n_seqs + 1] = row range of each sequence, kv_lens [n_seqs] = the sequence's length
+ * INCLUDING this step's rows (so a row's position is kv_lens[s] - (cu_q[s+1] - cu_q[s]) + its index in the
+ * range), slot_ids [n_seqs] = the sequence's recurrent-state slot.  A sequence whose first row is at position 0
+ * starts from a zero state whatever its slot holds. */
+
+/* y [M][N] (ldy) = alpha * x [M][K] (ldx) . w[N][K]^T, any M, N, K.  bf16 weights: x is rounded to bf16 and the
+ * product runs on MFMA (M > 8), unless exact != 0: then - and always for fp32 weights - x is not rounded and the
+ * sum over k is an fp32 FMA chain. */
+int mi_gemm_any(const float* x, int64_t ldx, const void* w, int w_dtype, float* y, int64_t ldy, int M, int N, int K,
+                float alpha, int exact, mi_stream stream);
+/* The same over groups of rows with one weight [N][K] each (w = [n_groups][N][K]): the rows of group g are the
+ * sorted positions [group_offsets[g], group_offsets[g+1]) (device memory; no group has more than
+ * rows_per_group_max); x row of position p = x_rows[p] (or p), y row = y_rows[p] (or p).  w2 != NULL:
+ * y = silu(x w^T) * (x w2^T). */
+int mi_gemm_any_grouped(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2, int w_dtype,
+                        const int32_t* group_offsets, int n_groups, int rows_per_group_max, float* y, int64_t ldy,
+                        const int32_t* y_rows, int N, int K, int exact, mi_stream stream);
+/* out[i] = table[ids[i]] widened to fp32. */
+int mi_embedding_f32(const int64_t* ids, const void* table, int table_dtype, float* out, int n, int width, int vocab,
+                     mi_stream stream);
+/* LayerNorm (mean and mean squared deviation in fp32, eps inside the root, weight and bias) of each row of y;
+ * add_to_out != 0: out += LN(y) (a residual stream whose norm sits on the sublayer's output). */
+int mi_layernorm_f32(const float* y, int64_t ldy, const float* w, const float* b, float* out, int64_t ldo, int rows,
+                     int width, float eps, int add_to_out, mi_stream stream);
+/* Sliding-window attention, per-row preparation.  proj rows hold q [H*D] at q_off, k [G*D] at k_off, v [G*Dv] at
+ * v_off.  q <- q / rms(q over ALL H*D) * qn_w in place; k likewise with kn_w, stored to k_cache; v_first != NULL:
+ * v <- (1 - *lam) v + *lam * v_first (in place), stored to v_cache.  Caches [blocks][G][block_size][D | Dv],
+ * slots[row] = block * block_size + offset, or < 0: not stored. */
+int mi_swa_prepare(float* proj, int64_t ld, int q_off, int k_off, int v_off, const float* qn_w, const float* kn_w,
+                   float eps, const float* v_first, int64_t ld_vf, const float* lam, void* k_cache, void* v_cache,
+                   int cache_dtype, const int32_t* slots, int rows, int H, int G, int D, int Dv, int block_size,
+                   mi_stream stream);
+/* out[row][h*Dv..] = softmax_j(scale q.k_j - 2^(-8 (h+1) / H) (i - j)) v_j over the keys 0 <= i - j < window of the
+ * row's sequence (all of which must be in the cache), times sigmoid(gate[row][h*Dv..]) if gate != NULL.
+ * Query head h reads kv head h / (H / G). */
+int mi_swa_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int cache_dtype,
+                     const int32_t* block_tables, int table_cols, const int32_t* cu_q, const int32_t* kv_lens,
+                     int n_seqs, int rows, int H, int G, int D, int Dv, int block_size, int window, float scale,
+                     const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream);
+/* y = silu(depthwise causal convolution of x over time), w [channels][taps] (last tap = the current row), the
+ * taps - 1 inputs before a step's first row taken from state [slots][taps - 1][channels] (oldest first).
+ * mi_causal_conv_state then writes the new tail (call it after every consumer of the old one). */
+int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, const float* state, const int32_t* cu_q,
+                        const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows, int channels, float* y,
+                        int64_t ldy, mi_stream stream);
+int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, const int32_t* cu_q,
+                         const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int channels, mi_stream stream);
+/* Gated delta rule with a decay per (head, key channel); state [slots][H][D][Dv] fp32.  Per row and head h (q / k
+ * head h / (H / G)): q, k <- unit vectors (x / sqrt(sum x^2 + 1e-6)), q / sqrt(D); g = exp(-exp(a_log[h]) *
+ * softplus(decay_pre[row][h*D..] + dt_bias[h*D..])); beta = sigmoid(beta_pre[row][h]);
+ * S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
+ * out = o / rms(o over Dv) * norm_w * sigmoid(gate_pre[row][h*Dv..]). */
+int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_off, const float* beta_pre,
+                     int64_t ld_beta, const float* decay_pre, int64_t ld_decay, const float* dt_bias,
+                     const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w, float* state,
+                     const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int H, int G,
+                     int D, int Dv, float eps, float* out, int64_t ldo, mi_stream stream);
+/* Router with expert groups: scores = softmax(logits) over n_outputs; choice = scores + correction; only the
+ * `keep` of `n_groups` equal groups of neighbours with the largest best choice are eligible; ids = the top_k
+ * eligible outputs by choice (descending), weights = their scores (not renormalised).  n_outputs <= 512. */
+int mi_route_grouped(const float* logits, int64_t ld, const float* correction, int n_tokens, int n_outputs, int top_k,
+                     int n_groups, int keep, int32_t* ids, float* weights, mi_stream stream);
+/* out[t] = sum_k weights[t][k] * (ids[t][k] >= n_experts ? h[t] : y[t * top_k + k]) in slot order. */
+int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, const int32_t* ids, const float* weights,
+                       int n_tokens, int top_k, int n_experts, int width, float* out, int64_t ldo, mi_stream stream);
+
 /* ---- host-side hashing (reference: engine/block_manager.py:38-44) --------- */
 /* xxh64 of `len` bytes with seed 0, optionally prefixed by the 8 little-endian
  * bytes of `prefix` (has_prefix != 0) — the chained block hash of

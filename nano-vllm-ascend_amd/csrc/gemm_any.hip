@@ -1,0 +1,326 @@
+// General-shape projections with fp32 activations: y = alpha * x . w^T for ANY M, N, K (no multiple-of-64 contract),
+// weights bf16 or fp32 as stored ([N][K] row-major), fp32 accumulation, fp32 output - plain, and grouped over
+// expert-sorted rows (one launch for all experts of a sparse feed-forward, SwiGLU optionally in the epilogue).
+//
+// These serve the model families whose residual stream, norms and recurrences are kept in 32-bit floats and whose
+// widths are not the fragment-native kernels' (csrc/gemm_skinny*.hpp, gemm_tile.hip): three kernels,
+//
+//   gemm_any_mfma_kernel   bf16 weights: 64 x 64 output tile per 4-wave workgroup, x rounded to bf16 on its way into
+//                          LDS, v_mfma_f32_16x16x32_bf16, edges zero-filled by guarded loads
+//   gemm_any_fma_kernel    true 32-bit: fp32 (or bf16, widened exactly) weights, x NOT rounded, plain FMA chains in k
+//                          order - the float32 serving mode, and the routers of sparse feed-forwards in either mode
+//   gemm_any_rows_kernel   M <= 8 rows (decode): one wave per output feature streams its weight row once, lanes
+//                          split K in 16-byte pieces, butterfly reduction; both dtypes, x not rounded
+//
+// A row of the result is a function of its own x row and the weights only: the summation order over k does not depend
+// on M, on the row's place in the batch or on the tile it falls into (each kernel has ONE fixed order), so the same
+// token gives the same bits whatever it is batched with, within one kernel; between kernels (a row computed in a
+// prompt's portion vs alone) results differ by rounding only.
+#include "mi_common.hpp"
+
+namespace mi {
+
+struct GemmAnyArgs {
+  const float* x;
+  int64_t ldx;
+  const void* w;    // [groups][N][K]
+  const void* w2;   // nullptr, or the second weight of the SwiGLU epilogue: y = silu(x w^T) * (x w2^T)
+  float* y;
+  int64_t ldy;
+  int M, N, K;
+  float alpha;
+  const int32_t* group_offsets;  // nullptr: one group of M rows; else rows of group g = [off[g], off[g + 1])
+  const int32_t* x_rows;         // nullptr or the x row of each (sorted) row
+  const int32_t* y_rows;         // nullptr or the y row of each (sorted) row
+};
+
+template <typename TW>
+__device__ __forceinline__ float w_load(const TW* p);
+template <>
+__device__ __forceinline__ float w_load<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float w_load<uint16_t>(const uint16_t* p) { return bf2f(*p); }
+
+__device__ __forceinline__ bool dev_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+
+// ---------------------------------------------------------------------------------------------------------------
+// exact kernel: 64 x 64 tile, 256 threads, 4 x 4 outputs per thread, k ascending
+// ---------------------------------------------------------------------------------------------------------------
+template <typename TW, bool DUAL>
+__global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
+  constexpr int BM = 64, BN = 64, BK = 32, PAD = 4;
+  __shared__ float As[BK][BM + PAD];
+  __shared__ float Bs[DUAL ? 2 : 1][BK][BN + PAD];
+  const int tid = threadIdx.x;
+  int m_lo = 0, m_hi = a.M;
+  const TW* w = static_cast<const TW*>(a.w);
+  const TW* w2 = static_cast<const TW*>(a.w2);
+  if (a.group_offsets) {
+    m_lo = a.group_offsets[blockIdx.z];
+    m_hi = a.group_offsets[blockIdx.z + 1];
+    w += (int64_t)blockIdx.z * a.N * a.K;
+    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
+  }
+  const int m0 = m_lo + blockIdx.y * BM;
+  if (m0 >= m_hi) return;
+  const int n0 = blockIdx.x * BN;
+  const int lr = tid >> 2, lk = (tid & 3) * 8;  // this thread stages 8 consecutive k of one row
+  int64_t xrow = -1;
+  if (m0 + lr < m_hi) xrow = a.x_rows ? a.x_rows[m0 + lr] : m0 + lr;
+  const int wrow = n0 + lr < a.N ? n0 + lr : -1;
+  float acc[DUAL ? 2 : 1][4][4] = {};
+  const int ty = tid >> 4, tx = tid & 15;
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int k = k0 + lk + i;
+      As[lk + i][lr] = (xrow >= 0 && k < a.K) ? a.x[xrow * a.ldx + k] : 0.f;
+      Bs[0][lk + i][lr] = (wrow >= 0 && k < a.K) ? w_load<TW>(w + (int64_t)wrow * a.K + k) : 0.f;
+      if (DUAL) Bs[1][lk + i][lr] = (wrow >= 0 && k < a.K) ? w_load<TW>(w2 + (int64_t)wrow * a.K + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < BK; ++k) {
+      float av[4], bv[DUAL ? 2 : 1][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bv[d][j] = Bs[d][k][tx * 4 + j];
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[d][i][j] = fmaf(av[i], bv[d][j], acc[d][i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= m_hi) continue;
+    const int64_t yrow = a.y_rows ? a.y_rows[m] : m;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= a.N) continue;
+      float v = acc[0][i][j];
+      if (DUAL) v = silu_f(v) * acc[1][i][j];
+      a.y[yrow * a.ldy + n] = v * a.alpha;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// MFMA kernel (bf16 weights): 64 x 64 tile, 4 waves as 2 x 2, each wave 32 x 32 = 2 x 2 fragments of 16 x 16,
+// K in steps of 32.  LDS holds the tile's x rows and weight rows as bf16 [64][32 + 8] (row stride 80 bytes: the eight
+// rows a quarter-wave reads start in different banks).
+// ---------------------------------------------------------------------------------------------------------------
+template <bool DUAL>
+__global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
+  constexpr int BM = 64, BN = 64, BK = 32, LD = BK + 8;
+  __shared__ __attribute__((aligned(16))) uint16_t As[BM][LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[DUAL ? 2 : 1][BN][LD];
+  const int tid = threadIdx.x;
+  int m_lo = 0, m_hi = a.M;
+  const uint16_t* w = static_cast<const uint16_t*>(a.w);
+  const uint16_t* w2 = static_cast<const uint16_t*>(a.w2);
+  if (a.group_offsets) {
+    m_lo = a.group_offsets[blockIdx.z];
+    m_hi = a.group_offsets[blockIdx.z + 1];
+    w += (int64_t)blockIdx.z * a.N * a.K;
+    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
+  }
+  const int m0 = m_lo + blockIdx.y * BM;
+  if (m0 >= m_hi) return;
+  const int n0 = blockIdx.x * BN;
+  const int lr = tid >> 2, lk = (tid & 3) * 8;
+  int64_t xrow = -1;
+  if (m0 + lr < m_hi) xrow = a.x_rows ? a.x_rows[m0 + lr] : m0 + lr;
+  const int wrow = n0 + lr < a.N ? n0 + lr : -1;
+  const bool w_vec = (a.K % 8 == 0) && dev_aligned16(a.w) && (!DUAL || dev_aligned16(a.w2));
+  const bool x_vec = (a.ldx % 4 == 0) && dev_aligned16(a.x);
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int fr = lane & 15, fk = (lane >> 4) * 8;
+  f32x4 acc[DUAL ? 2 : 1][2][2];
+#pragma unroll
+  for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[d][i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    const int k = k0 + lk;
+    // x: 8 floats -> 8 bf16 (round to nearest even)
+    float xv[8];
+    if (xrow >= 0 && x_vec && k + 8 <= a.K) {
+      const float4 p0 = *reinterpret_cast<const float4*>(a.x + xrow * a.ldx + k);
+      const float4 p1 = *reinterpret_cast<const float4*>(a.x + xrow * a.ldx + k + 4);
+      xv[0] = p0.x, xv[1] = p0.y, xv[2] = p0.z, xv[3] = p0.w, xv[4] = p1.x, xv[5] = p1.y, xv[6] = p1.z, xv[7] = p1.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xv[i] = (xrow >= 0 && k + i < a.K) ? a.x[xrow * a.ldx + k + i] : 0.f;
+    }
+    u32x4 xp = {pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
+    *reinterpret_cast<u32x4*>(&As[lr][lk]) = xp;
+#pragma unroll
+    for (int d = 0; d < (DUAL ? 2 : 1); ++d) {
+      const uint16_t* wp = (d ? w2 : w) + (int64_t)wrow * a.K + k;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (wrow >= 0) {
+        if (w_vec && k + 8 <= a.K) {
+          v = *reinterpret_cast<const u32x4*>(wp);
+        } else {
+          uint16_t e[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) e[i] = k + i < a.K ? wp[i] : (uint16_t)0;
+          v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                    (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+        }
+      }
+      *reinterpret_cast<u32x4*>(&Bs[d][lr][lk]) = v;
+    }
+    __syncthreads();
+    bf16x8 af[2], bfr[DUAL ? 2 : 1][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) af[i] = as_frag(*reinterpret_cast<const u32x4*>(&As[wm + i * 16 + fr][fk]));
+#pragma unroll
+    for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bfr[d][j] = as_frag(*reinterpret_cast<const u32x4*>(&Bs[d][wn + j * 16 + fr][fk]));
+    // D[n][m] = sum_k W[n][k] X[m][k]: weights on the MFMA's row axis, so a lane's four results are four consecutive
+    // FEATURES of one x row
+#pragma unroll
+    for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[d][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[d][j], af[i], acc[d][i][j], 0, 0, 0);
+    __syncthreads();
+  }
+  // fragment (i, j): x row = wm + i*16 + (lane & 15), features wn + j*16 + (lane >> 4) * 4 + r
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = m0 + wm + i * 16 + (lane & 15);
+    if (m >= m_hi) continue;
+    const int64_t yrow = a.y_rows ? a.y_rows[m] : m;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = n0 + wn + j * 16 + (lane >> 4) * 4 + r;
+        if (n >= a.N) continue;
+        float v = acc[0][i][j][r];
+        if (DUAL) v = silu_f(v) * acc[1][i][j][r];
+        a.y[yrow * a.ldy + n] = v * a.alpha;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// few rows (decode): one wave per output feature; lanes take K in pieces of 8, ascending, then a butterfly
+// ---------------------------------------------------------------------------------------------------------------
+template <typename TW, int MT, bool DUAL>
+__global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  int m_lo = 0, m_hi = a.M;
+  const TW* w = static_cast<const TW*>(a.w);
+  const TW* w2 = static_cast<const TW*>(a.w2);
+  if (a.group_offsets) {
+    m_lo = a.group_offsets[blockIdx.z];
+    m_hi = a.group_offsets[blockIdx.z + 1];
+    w += (int64_t)blockIdx.z * a.N * a.K;
+    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
+  }
+  if (n >= a.N) return;  // (whole waves: the reductions below see all 64 lanes)
+  for (int m0 = m_lo; m0 < m_hi; m0 += MT) {
+    float acc[DUAL ? 2 : 1][MT] = {};
+    int64_t xr[MT];
+#pragma unroll
+    for (int r = 0; r < MT; ++r) xr[r] = m0 + r < m_hi ? (a.x_rows ? a.x_rows[m0 + r] : m0 + r) : -1;
+    for (int k0 = lane * 8; k0 < a.K; k0 += 64 * 8) {
+      float wv[DUAL ? 2 : 1][8];
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          wv[d][i] = k0 + i < a.K ? w_load<TW>((d ? w2 : w) + (int64_t)n * a.K + k0 + i) : 0.f;
+#pragma unroll
+      for (int r = 0; r < MT; ++r) {
+        if (xr[r] < 0) continue;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xv = k0 + i < a.K ? a.x[xr[r] * a.ldx + k0 + i] : 0.f;
+#pragma unroll
+          for (int d = 0; d < (DUAL ? 2 : 1); ++d) acc[d][r] = fmaf(xv, wv[d][i], acc[d][r]);
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < MT; ++r) {
+      float v = wave_sum(acc[0][r]);
+      if (DUAL) v = silu_f(v) * wave_sum(acc[1][r]);
+      if (lane == 0 && xr[r] >= 0) {
+        const int64_t yrow = a.y_rows ? a.y_rows[m0 + r] : m0 + r;
+        a.y[yrow * a.ldy + n] = v * a.alpha;
+      }
+    }
+  }
+}
+
+template <typename TW, bool DUAL>
+static int launch_any(const GemmAnyArgs& a, int groups, int rows_per_group_max, int mode, hipStream_t st) {
+  // mode 0: product (MFMA for bf16 weights, the row kernel for few rows); 1: exact (FMA chains / row kernel, x unrounded)
+  if (rows_per_group_max <= 8) {
+    const dim3 grid((a.N + 3) / 4, 1, groups);
+    if (rows_per_group_max <= 1) hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 1, DUAL>), grid, dim3(256), 0, st, a);
+    else if (rows_per_group_max <= 4) hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 4, DUAL>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 8, DUAL>), grid, dim3(256), 0, st, a);
+    return check_launch();
+  }
+  const dim3 grid((a.N + 63) / 64, (rows_per_group_max + 63) / 64, groups);
+  if constexpr (sizeof(TW) == 2) {
+    if (mode == 0) {
+      hipLaunchKernelGGL((gemm_any_mfma_kernel<DUAL>), grid, dim3(256), 0, st, a);
+      return check_launch();
+    }
+  }
+  hipLaunchKernelGGL((gemm_any_fma_kernel<TW, DUAL>), grid, dim3(256), 0, st, a);
+  return check_launch();
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+static int gemm_any_dispatch(const GemmAnyArgs& a, int w_dtype, int groups, int rows_max, int mode, hipStream_t st) {
+  if (a.M == 0 || a.N == 0 || rows_max == 0) return MI_OK;
+  if (w_dtype == MI_DTYPE_BF16)
+    return a.w2 ? launch_any<uint16_t, true>(a, groups, rows_max, mode, st) : launch_any<uint16_t, false>(a, groups, rows_max, mode, st);
+  if (w_dtype == MI_DTYPE_F32)
+    return a.w2 ? launch_any<float, true>(a, groups, rows_max, mode, st) : launch_any<float, false>(a, groups, rows_max, mode, st);
+  return MI_EINVAL;
+}
+
+extern "C" int mi_gemm_any(const float* x, int64_t ldx, const void* w, int w_dtype, float* y, int64_t ldy, int M, int N,
+                           int K, float alpha, int exact, mi_stream stream) {
+  if (!x || !w || !y || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N) return MI_EINVAL;
+  GemmAnyArgs a{x, ldx, w, nullptr, y, ldy, M, N, K, alpha, nullptr, nullptr, nullptr};
+  return gemm_any_dispatch(a, w_dtype, 1, M, exact ? 1 : 0, S(stream));
+}
+
+extern "C" int mi_gemm_any_grouped(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2,
+                                   int w_dtype, const int32_t* group_offsets, int n_groups, int rows_per_group_max,
+                                   float* y, int64_t ldy, const int32_t* y_rows, int N, int K, int exact,
+                                   mi_stream stream) {
+  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1) return MI_EINVAL;
+  if (n_groups > 65535) return MI_EUNSUPPORTED;
+  GemmAnyArgs a{x, ldx, w, w2, y, ldy, rows_per_group_max, N, K, 1.0f, group_offsets, x_rows, y_rows};
+  return gemm_any_dispatch(a, w_dtype, n_groups, rows_per_group_max, exact ? 1 : 0, S(stream));
+}

@@ -1,0 +1,560 @@
+// Sequence mixers and row operators of the model families that keep their residual stream in 32-bit floats:
+//
+//   mi_embedding_f32            table rows (bf16 or fp32) -> fp32 residual rows
+//   mi_layernorm_f32            LayerNorm with weight and bias; optionally ADDED to a residual in place
+//                               (x <- x + LN(y): the norm sits on the sublayer's output)
+//   mi_swa_prepare              sliding-window attention, K/V side: ONE root-mean-square norm over a token's whole q
+//                               projection and one over its whole k projection (not per head), optional mixing of the
+//                               values with an earlier layer's values of the same token, K / V rows to the paged cache
+//   mi_swa_attention            paged sliding-window attention with a per-head linear distance bias
+//                               s_ij = scale q_i.k_j - slope_h (i - j), keys 0 <= i - j < window, separate key and value
+//                               head sizes, grouped heads, optional sigmoid output gate; prompt portions and single
+//                               decoded tokens in one launch (a row's keys are addressed through its sequence's block
+//                               table and total length)
+//   mi_causal_conv_silu         short causal depthwise convolution over time + SiLU, carried across steps by a
+//   mi_causal_conv_state        per-sequence state slot holding the last taps - 1 inputs
+//   mi_channel_delta            gated delta rule with one decay per head AND key channel:
+//                               S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
+//                               with unit-norm q / k, per-head RMS norm of o, sigmoid gate; the fp32 state lives in a
+//                               per-sequence slot and is carried from step to step
+//   mi_route_grouped            router of a sparse feed-forward: softmax scores, additive choice correction, choice
+//                               restricted to the best groups of experts, top-k; weights = un-renormalised scores
+//   mi_moe_combine_f32          out[t] = sum_k w[t][k] * (identity expert ? h[t] : y[t * top_k + k])
+//
+// Everything here is computed in fp32 (expf / logf / sqrtf of the device library, no fast-math), for both serving
+// dtypes: the bf16 mode differs only in the dtype of the WEIGHTS and of the K/V cache.
+// A step's rows are described by cu_q [n_seqs + 1] (row range of each sequence) and kv_lens [n_seqs] (the sequence's
+// length INCLUDING this step's rows): row r of sequence s sits at position kv_lens[s] - (cu_q[s+1] - cu_q[s]) + r.
+#include "mi_common.hpp"
+
+namespace mi {
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+template <typename T>
+__device__ __forceinline__ float ld_f(const T* p);
+template <>
+__device__ __forceinline__ float ld_f<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float ld_f<uint16_t>(const uint16_t* p) { return bf2f(*p); }
+template <typename T>
+__device__ __forceinline__ void st_f(T* p, float v);
+template <>
+__device__ __forceinline__ void st_f<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void st_f<uint16_t>(uint16_t* p, float v) { *p = f2bf(v); }
+
+// sum over a 256-thread workgroup; every thread gets the result.  red: 4 floats of LDS per concurrent reduction.
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();  // (red may still be read from the previous reduction)
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// the sequence a step row belongs to (n_seqs is small: a linear walk, identical on every lane)
+__device__ __forceinline__ int seq_of_row(const int32_t* cu_q, int n_seqs, int row) {
+  int s = 0;
+  while (s + 1 < n_seqs && row >= cu_q[s + 1]) ++s;
+  return s;
+}
+
+template <typename TT>
+__global__ __launch_bounds__(256) void embedding_f32_kernel(const int64_t* __restrict__ ids, const TT* __restrict__ table,
+                                                            float* __restrict__ out, int width, int vocab) {
+  const int64_t id = ids[blockIdx.x];
+  if (id < 0 || id >= vocab) return;
+  for (int c = threadIdx.x; c < width; c += 256) out[(int64_t)blockIdx.x * width + c] = ld_f<TT>(table + id * width + c);
+}
+
+// one workgroup per row; mean, then the mean of squared deviations (two passes over the row, which stays in L1)
+__global__ __launch_bounds__(256) void layernorm_f32_kernel(const float* __restrict__ y, int64_t ldy,
+                                                            const float* __restrict__ w, const float* __restrict__ b,
+                                                            float* __restrict__ out, int64_t ldo, int width, float eps,
+                                                            int add) {
+  __shared__ float red[4];
+  const float* yr = y + (int64_t)blockIdx.x * ldy;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) s += yr[c];
+  const float mean = block_sum256(s, red) / (float)width;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float d = yr[c] - mean;
+    q += d * d;
+  }
+  const float var = block_sum256(q, red) / (float)width;
+  const float rstd = 1.f / sqrtf(var + eps);
+  float* o = out + (int64_t)blockIdx.x * ldo;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = (yr[c] - mean) * rstd * w[c] + b[c];
+    o[c] = add ? o[c] + v : v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// sliding-window attention
+// ---------------------------------------------------------------------------------------------------------------
+// One workgroup per step row.  q (qn values at proj + q_off) is normalised in place; k is normalised and stored; v is
+// mixed (written back in place, so that a later layer can take it as ITS v_first only if this layer is the first mixing
+// one - the caller keeps that tensor) and stored.  Cache layout [blocks][kv heads][block][dim], slot = block * block_size
+// + offset, slot < 0: not stored.
+template <typename TC>
+__global__ __launch_bounds__(256) void swa_prepare_kernel(float* __restrict__ proj, int64_t ld, int q_off, int k_off,
+                                                          int v_off, int nq, int nk, int nv,
+                                                          const float* __restrict__ qn_w, const float* __restrict__ kn_w,
+                                                          float eps, const float* __restrict__ v_first, int64_t ld_vf,
+                                                          const float* __restrict__ lam_p, TC* __restrict__ k_cache,
+                                                          TC* __restrict__ v_cache, const int32_t* __restrict__ slots,
+                                                          int G, int D, int Dv, int block_size) {
+  __shared__ float red[4];
+  float* row = proj + (int64_t)blockIdx.x * ld;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x; c < nq; c += 256) sq += row[q_off + c] * row[q_off + c];
+  for (int c = threadIdx.x; c < nk; c += 256) sk += row[k_off + c] * row[k_off + c];
+  const float rq = 1.f / sqrtf(block_sum256(sq, red) / (float)nq + eps);
+  const float rk = 1.f / sqrtf(block_sum256(sk, red) / (float)nk + eps);
+  for (int c = threadIdx.x; c < nq; c += 256) row[q_off + c] = row[q_off + c] * rq * qn_w[c];
+  const int slot = slots[blockIdx.x];
+  const int64_t blk = slot >= 0 ? slot / block_size : 0;
+  const int off = slot >= 0 ? slot % block_size : 0;
+  for (int c = threadIdx.x; c < nk; c += 256) {
+    const float v = row[k_off + c] * rk * kn_w[c];
+    if (slot >= 0) st_f<TC>(k_cache + ((blk * G + c / D) * block_size + off) * D + c % D, v);
+  }
+  const float lam = (v_first && lam_p) ? *lam_p : 0.f;
+  for (int c = threadIdx.x; c < nv; c += 256) {
+    float v = row[v_off + c];
+    if (v_first) {
+      v = (1.f - lam) * v + lam * v_first[(int64_t)blockIdx.x * ld_vf + c];
+      row[v_off + c] = v;
+    }
+    if (slot >= 0) st_f<TC>(v_cache + ((blk * G + c / Dv) * block_size + off) * Dv + c % Dv, v);
+  }
+}
+
+// One wave per (row, head); lanes over keys for the scores, over value channels for the output.
+template <typename TC, int VPL>  // VPL: value channels per lane (Dv <= 64 * VPL)
+__global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restrict__ q, int64_t ldq,
+                                                            const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
+                                                            const int32_t* __restrict__ block_tables, int table_cols,
+                                                            const int32_t* __restrict__ cu_q,
+                                                            const int32_t* __restrict__ kv_lens, int n_seqs, int n_rows,
+                                                            int H, int G, int D, int Dv, int block_size, int window,
+                                                            float scale, const float* __restrict__ gate, int64_t ldg,
+                                                            float* __restrict__ out, int64_t ldo) {
+  extern __shared__ float smem[];  // per wave: q [D], p [64]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wid = blockIdx.x * 4 + wave;
+  if (wid >= n_rows * H) return;
+  const int row = wid / H, h = wid % H;
+  float* qs = smem + wave * (D + 64);
+  float* ps = qs + D;
+  for (int d = lane; d < D; d += 64) qs[d] = q[(int64_t)row * ldq + h * D + d];
+  const int s = seq_of_row(cu_q, n_seqs, row);
+  const int pos = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (row - cu_q[s]);
+  const int lo = max(0, pos - window + 1);
+  const int g = h / (H / G);
+  const float slope = exp2f(-8.f * (float)(h + 1) / (float)H);
+  const int32_t* table = block_tables + (int64_t)s * table_cols;
+  float m = -INFINITY, l = 0.f;
+  float acc[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) acc[i] = 0.f;
+  __builtin_amdgcn_wave_barrier();
+  for (int j0 = lo; j0 <= pos; j0 += 64) {
+    const int j = j0 + lane;
+    float sc = -INFINITY;
+    if (j <= pos) {
+      const int64_t blk = table[j / block_size];
+      const TC* kr = k_cache + ((blk * G + g) * block_size + j % block_size) * D;
+      float dot = 0.f;
+      for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld_f<TC>(kr + d), dot);
+      sc = dot * scale - slope * (float)(pos - j);
+    }
+    const float m_new = fmaxf(m, wave_max(sc));
+    const float p = j <= pos ? expf(sc - m_new) : 0.f;
+    const float corr = expf(m - m_new);  // (first chunk: exp(-inf) = 0)
+    l = l * corr + wave_sum(p);
+    m = m_new;
+    ps[lane] = p;
+    __builtin_amdgcn_wave_barrier();
+    const int n_keys = min(64, pos - j0 + 1);
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) acc[i] *= corr;
+    for (int jj = 0; jj < n_keys; ++jj) {
+      const int jk = j0 + jj;
+      const int64_t blk = table[jk / block_size];
+      const TC* vr = v_cache + ((blk * G + g) * block_size + jk % block_size) * Dv;
+      const float pj = ps[jj];
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int d = lane + 64 * i;
+        if (d < Dv) acc[i] = fmaf(pj, ld_f<TC>(vr + d), acc[i]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float inv = 1.f / l;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int d = lane + 64 * i;
+    if (d < Dv) {
+      float o = acc[i] * inv;
+      if (gate) o *= sigmoid_f(gate[(int64_t)row * ldg + h * Dv + d]);
+      out[(int64_t)row * ldo + h * Dv + d] = o;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// short causal convolution with a carried tail
+// ---------------------------------------------------------------------------------------------------------------
+// y[r][c] = silu(sum_j w[c][j] * in[r - (taps - 1) + j]); inputs before the step's first row come from the sequence's
+// state slot (the last taps - 1 inputs, oldest first) - zeros when the sequence starts in this step.
+__global__ __launch_bounds__(256) void causal_conv_silu_kernel(const float* __restrict__ x, int64_t ldx,
+                                                               const float* __restrict__ w, int taps,
+                                                               const float* __restrict__ state,
+                                                               const int32_t* __restrict__ cu_q,
+                                                               const int32_t* __restrict__ kv_lens,
+                                                               const int32_t* __restrict__ slot_ids, int n_seqs, int C,
+                                                               float* __restrict__ y, int64_t ldy) {
+  const int row = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int s = seq_of_row(cu_q, n_seqs, row);
+  const int r = row - cu_q[s];
+  const int start = kv_lens[s] - (cu_q[s + 1] - cu_q[s]);
+  const float* st = state + (int64_t)slot_ids[s] * (taps - 1) * C;
+  float acc = 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int rr = r - (taps - 1) + j;  // row of this sequence's step, or before it
+    float v;
+    if (rr >= 0) v = x[(int64_t)(cu_q[s] + rr) * ldx + c];
+    else v = start > 0 ? st[(int64_t)(taps - 1 + rr) * C + c] : 0.f;  // (a state written at position p holds inputs p-taps+1..p-1, zeros before 0)
+    acc = fmaf(w[(int64_t)c * taps + j], v, acc);
+  }
+  y[(int64_t)row * ldy + c] = acc / (1.f + expf(-acc));
+}
+
+// the new tail: the last taps - 1 inputs of (old tail ++ this step's rows).  One thread per (sequence, channel) reads
+// everything it needs before it writes, and no other thread touches its entries.
+__global__ __launch_bounds__(256) void causal_conv_state_kernel(const float* __restrict__ x, int64_t ldx, int taps,
+                                                                float* __restrict__ state,
+                                                                const int32_t* __restrict__ cu_q,
+                                                                const int32_t* __restrict__ kv_lens,
+                                                                const int32_t* __restrict__ slot_ids, int C) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int n = cu_q[s + 1] - cu_q[s];
+  if (n == 0) return;
+  const int start = kv_lens[s] - n;
+  float* st = state + (int64_t)slot_ids[s] * (taps - 1) * C;
+  float tail[16];
+  const int L = taps - 1;
+  for (int i = 0; i < L; ++i) {
+    const int rr = n - L + i;  // row of this step, or (negative) an entry of the old tail
+    if (rr >= 0) tail[i] = x[(int64_t)(cu_q[s] + rr) * ldx + c];
+    else tail[i] = start > 0 ? st[(int64_t)(L + rr) * C + c] : 0.f;
+  }
+  for (int i = 0; i < L; ++i) st[(int64_t)i * C + c] = tail[i];
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// gated delta rule, decay per head and key channel
+// ---------------------------------------------------------------------------------------------------------------
+// One workgroup per (sequence, head), walking the sequence's rows of this step in order.  The state S [D][Dv] stays in
+// LDS for the whole walk (thread j owns column j: S^T k, the rank-one update and S^T q are per-column loops without any
+// exchange), read from / written to the sequence's slot.  Threads i < D prepare the row's key-channel vectors (unit q
+// and k, decay), threads j < Dv the value side.  blockDim = max(D, Dv) rounded up to 64.
+__global__ void channel_delta_kernel(const float* __restrict__ qkv, int64_t ld, int q_off, int k_off, int v_off,
+                                     const float* __restrict__ beta_pre, int64_t ld_beta,
+                                     const float* __restrict__ decay_pre, int64_t ld_decay,
+                                     const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                                     const float* __restrict__ gate_pre, int64_t ld_gate,
+                                     const float* __restrict__ norm_w, float* __restrict__ state,
+                                     const int32_t* __restrict__ cu_q, const int32_t* __restrict__ kv_lens,
+                                     const int32_t* __restrict__ slot_ids, int H, int G, int D, int Dv, float eps,
+                                     float* __restrict__ out, int64_t ldo) {
+  extern __shared__ float smem[];
+  float* S = smem;                 // [D][Dv]
+  float* qv = S + D * Dv;          // [D]
+  float* kv = qv + D;              // [D]
+  float* gv = kv + D;              // [D]
+  float* red = gv + D;             // [16]
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, nthr = blockDim.x, nwaves = nthr >> 6;
+  const int r0 = cu_q[s], n = cu_q[s + 1] - r0;
+  if (n == 0) return;
+  const int start = kv_lens[s] - n;
+  const int kvh = h / (H / G);
+  float* slot = state + ((int64_t)slot_ids[s] * H + h) * D * Dv;
+  for (int e = tid; e < D * Dv; e += nthr) S[e] = start > 0 ? slot[e] : 0.f;
+  const float decay_rate = expf(a_log[h]);
+  const float q_scale = 1.f / sqrtf((float)D);
+  __syncthreads();
+  for (int r = 0; r < n; ++r) {
+    const int64_t row = r0 + r;
+    // key side: sums of squares of q and k over D (fixed order: wave butterfly, then the waves in order)
+    float qr = 0.f, kr = 0.f;
+    if (tid < D) {
+      qr = qkv[row * ld + q_off + kvh * D + tid];
+      kr = qkv[row * ld + k_off + kvh * D + tid];
+    }
+    const float sq = wave_sum(qr * qr), sk = wave_sum(kr * kr);
+    if ((tid & 63) == 0) red[tid >> 6] = sq, red[8 + (tid >> 6)] = sk;
+    __syncthreads();
+    float tq = 0.f, tk = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) tq += red[wv], tk += red[8 + wv];
+    if (tid < D) {
+      qv[tid] = qr / sqrtf(tq + 1e-6f) * q_scale;
+      kv[tid] = kr / sqrtf(tk + 1e-6f);
+      const float dt = softplus_f(decay_pre[row * ld_decay + h * D + tid] + dt_bias[h * D + tid]);
+      gv[tid] = expf(-decay_rate * dt);
+    }
+    __syncthreads();
+    float o = 0.f;
+    if (tid < Dv) {
+      float dot = 0.f;
+      for (int i = 0; i < D; ++i) {
+        const float sv = S[i * Dv + tid] * gv[i];
+        S[i * Dv + tid] = sv;
+        dot = fmaf(sv, kv[i], dot);
+      }
+      const float beta = sigmoid_f(beta_pre[row * ld_beta + h]);
+      const float u = beta * (qkv[row * ld + v_off + h * Dv + tid] - dot);
+      for (int i = 0; i < D; ++i) {
+        const float sv = fmaf(kv[i], u, S[i * Dv + tid]);
+        S[i * Dv + tid] = sv;
+        o = fmaf(sv, qv[i], o);
+      }
+    }
+    const float so = wave_sum(o * o);
+    __syncthreads();  // (red's previous contents have been read by everyone; qv / kv / gv are free again after this)
+    if ((tid & 63) == 0) red[tid >> 6] = so;
+    __syncthreads();
+    float to = 0.f;
+    for (int wv = 0; wv < nwaves; ++wv) to += red[wv];
+    if (tid < Dv) {
+      const float rstd = 1.f / sqrtf(to / (float)Dv + eps);
+      out[row * ldo + h * Dv + tid] = o * rstd * norm_w[tid] * sigmoid_f(gate_pre[row * ld_gate + h * Dv + tid]);
+    }
+    __syncthreads();
+  }
+  for (int e = tid; e < D * Dv; e += nthr) slot[e] = S[e];
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// sparse feed-forward: routing and combination
+// ---------------------------------------------------------------------------------------------------------------
+// One thread per token (n <= 512 router outputs, walked from global memory: the logits row is a few cache lines).
+__global__ __launch_bounds__(64) void route_grouped_kernel(const float* __restrict__ logits, int64_t ld,
+                                                           const float* __restrict__ correction, int T, int n, int top_k,
+                                                           int n_groups, int keep, int32_t* __restrict__ ids,
+                                                           float* __restrict__ wts) {
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t >= T) return;
+  const float* z = logits + (int64_t)t * ld;
+  float mx = -INFINITY;
+  for (int e = 0; e < n; ++e) mx = fmaxf(mx, z[e]);
+  float sum = 0.f;
+  for (int e = 0; e < n; ++e) sum += expf(z[e] - mx);
+  const int per = n / n_groups;
+  // groups kept: `keep` times the best remaining group (score = its largest choice score; ties: the lower index)
+  uint64_t kept[8] = {};  // n_groups <= 512
+  for (int it = 0; it < keep; ++it) {
+    int best = -1;
+    float best_v = -INFINITY;
+    for (int gi = 0; gi < n_groups; ++gi) {
+      if (kept[gi >> 6] >> (gi & 63) & 1) continue;
+      float gv = -INFINITY;
+      for (int e = gi * per; e < (gi + 1) * per; ++e) gv = fmaxf(gv, expf(z[e] - mx) / sum + correction[e]);
+      if (best < 0 || gv > best_v) best = gi, best_v = gv;
+    }
+    kept[best >> 6] |= 1ull << (best & 63);
+  }
+  uint64_t taken[8] = {};  // n <= 512
+  for (int it = 0; it < top_k; ++it) {
+    int best = -1;
+    float best_v = -INFINITY, best_s = 0.f;
+    for (int e = 0; e < n; ++e) {
+      const int gi = e / per;
+      if (!(kept[gi >> 6] >> (gi & 63) & 1) || (taken[e >> 6] >> (e & 63) & 1)) continue;
+      const float sc = expf(z[e] - mx) / sum;
+      const float ch = sc + correction[e];
+      if (best < 0 || ch > best_v) best = e, best_v = ch, best_s = sc;
+    }
+    taken[best >> 6] |= 1ull << (best & 63);
+    ids[(int64_t)t * top_k + it] = best;
+    wts[(int64_t)t * top_k + it] = best_s;
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_f32_kernel(const float* __restrict__ y, const float* __restrict__ h,
+                                                              int64_t ldh, const int32_t* __restrict__ ids,
+                                                              const float* __restrict__ wts, int top_k, int n_experts,
+                                                              int width, float* __restrict__ out, int64_t ldo) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float acc = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+      const int e = ids[(int64_t)t * top_k + k];
+      const float v = e >= n_experts ? h[(int64_t)t * ldh + c] : y[((int64_t)t * top_k + k) * width + c];
+      acc = fmaf(wts[(int64_t)t * top_k + k], v, acc);
+    }
+    out[(int64_t)t * ldo + c] = acc;
+  }
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" int mi_embedding_f32(const int64_t* ids, const void* table, int table_dtype, float* out, int n, int width,
+                                int vocab, mi_stream stream) {
+  if (!ids || !table || !out || n < 0 || width < 1) return MI_EINVAL;
+  if (n == 0) return MI_OK;
+  if (table_dtype == MI_DTYPE_BF16)
+    hipLaunchKernelGGL((embedding_f32_kernel<uint16_t>), dim3(n), dim3(256), 0, S(stream), ids,
+                       static_cast<const uint16_t*>(table), out, width, vocab);
+  else if (table_dtype == MI_DTYPE_F32)
+    hipLaunchKernelGGL((embedding_f32_kernel<float>), dim3(n), dim3(256), 0, S(stream), ids,
+                       static_cast<const float*>(table), out, width, vocab);
+  else return MI_EINVAL;
+  return check_launch();
+}
+
+extern "C" int mi_layernorm_f32(const float* y, int64_t ldy, const float* w, const float* b, float* out, int64_t ldo,
+                                int rows, int width, float eps, int add_to_out, mi_stream stream) {
+  if (!y || !w || !b || !out || rows < 0 || width < 1 || ldy < width || ldo < width) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  hipLaunchKernelGGL(layernorm_f32_kernel, dim3(rows), dim3(256), 0, S(stream), y, ldy, w, b, out, ldo, width, eps,
+                     add_to_out);
+  return check_launch();
+}
+
+extern "C" int mi_swa_prepare(float* proj, int64_t ld, int q_off, int k_off, int v_off, const float* qn_w,
+                              const float* kn_w, float eps, const float* v_first, int64_t ld_vf, const float* lam,
+                              void* k_cache, void* v_cache, int cache_dtype, const int32_t* slots, int rows, int H,
+                              int G, int D, int Dv, int block_size, mi_stream stream) {
+  if (!proj || !qn_w || !kn_w || !k_cache || !v_cache || !slots || rows < 0) return MI_EINVAL;
+  if (H < 1 || G < 1 || D < 1 || Dv < 1 || block_size < 1 || (v_first && !lam)) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  if (cache_dtype == MI_DTYPE_BF16)
+    hipLaunchKernelGGL((swa_prepare_kernel<uint16_t>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, k_off,
+                       v_off, H * D, G * D, G * Dv, qn_w, kn_w, eps, v_first, ld_vf, lam,
+                       static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(v_cache), slots, G, D, Dv, block_size);
+  else if (cache_dtype == MI_DTYPE_F32)
+    hipLaunchKernelGGL((swa_prepare_kernel<float>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, k_off, v_off,
+                       H * D, G * D, G * Dv, qn_w, kn_w, eps, v_first, ld_vf, lam, static_cast<float*>(k_cache),
+                       static_cast<float*>(v_cache), slots, G, D, Dv, block_size);
+  else return MI_EINVAL;
+  return check_launch();
+}
+
+template <typename TC>
+static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* vc, const int32_t* bt, int cols,
+                      const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
+                      int block_size, int window, float scale, const float* gate, int64_t ldg, float* out, int64_t ldo,
+                      hipStream_t st) {
+  const dim3 grid((rows * H + 3) / 4), block(256);
+  const size_t lds = 4 * (size_t)(D + 64) * sizeof(float);
+  const TC* k = static_cast<const TC*>(kc);
+  const TC* v = static_cast<const TC*>(vc);
+#define MI_SWA(VPL)                                                                                                  \
+  hipLaunchKernelGGL((swa_attention_kernel<TC, VPL>), grid, block, lds, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,     \
+                     n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo)
+  if (Dv <= 64) MI_SWA(1);
+  else if (Dv <= 128) MI_SWA(2);
+  else MI_SWA(4);
+#undef MI_SWA
+  return check_launch();
+}
+
+extern "C" int mi_swa_attention(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int cache_dtype,
+                                const int32_t* block_tables, int table_cols, const int32_t* cu_q, const int32_t* kv_lens,
+                                int n_seqs, int rows, int H, int G, int D, int Dv, int block_size, int window,
+                                float scale, const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream) {
+  if (!q || !k_cache || !v_cache || !block_tables || !cu_q || !kv_lens || !out || rows < 0 || n_seqs < 1) return MI_EINVAL;
+  if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1 || block_size < 1 || window < 1 || table_cols < 1) return MI_EINVAL;
+  if (Dv > 256 || D > 4096) return MI_EUNSUPPORTED;
+  if (rows == 0) return MI_OK;
+  if (cache_dtype == MI_DTYPE_BF16)
+    return launch_swa<uint16_t>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D,
+                                Dv, block_size, window, scale, gate, ldg, out, ldo, S(stream));
+  if (cache_dtype == MI_DTYPE_F32)
+    return launch_swa<float>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv,
+                             block_size, window, scale, gate, ldg, out, ldo, S(stream));
+  return MI_EINVAL;
+}
+
+extern "C" int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, const float* state,
+                                   const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs,
+                                   int rows, int channels, float* y, int64_t ldy, mi_stream stream) {
+  if (!x || !w || !state || !cu_q || !kv_lens || !slot_ids || !y || rows < 0 || n_seqs < 1 || channels < 1) return MI_EINVAL;
+  if (taps < 1 || taps > 17) return MI_EUNSUPPORTED;
+  if (rows == 0) return MI_OK;
+  if (rows > 65535) return MI_EUNSUPPORTED;
+  hipLaunchKernelGGL(causal_conv_silu_kernel, dim3((channels + 255) / 256, rows), dim3(256), 0, S(stream), x, ldx, w,
+                     taps, state, cu_q, kv_lens, slot_ids, n_seqs, channels, y, ldy);
+  return check_launch();
+}
+
+extern "C" int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, const int32_t* cu_q,
+                                    const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int channels,
+                                    mi_stream stream) {
+  if (!x || !state || !cu_q || !kv_lens || !slot_ids || n_seqs < 1 || channels < 1) return MI_EINVAL;
+  if (taps < 1 || taps > 17) return MI_EUNSUPPORTED;
+  if (taps == 1) return MI_OK;
+  hipLaunchKernelGGL(causal_conv_state_kernel, dim3((channels + 255) / 256, n_seqs), dim3(256), 0, S(stream), x, ldx,
+                     taps, state, cu_q, kv_lens, slot_ids, channels);
+  return check_launch();
+}
+
+extern "C" int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_off, const float* beta_pre,
+                                int64_t ld_beta, const float* decay_pre, int64_t ld_decay, const float* dt_bias,
+                                const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w,
+                                float* state, const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids,
+                                int n_seqs, int H, int G, int D, int Dv, float eps, float* out, int64_t ldo,
+                                mi_stream stream) {
+  if (!qkv || !beta_pre || !decay_pre || !dt_bias || !a_log || !gate_pre || !norm_w || !state || !cu_q || !kv_lens ||
+      !slot_ids || !out || n_seqs < 1)
+    return MI_EINVAL;
+  if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1) return MI_EINVAL;
+  const int threads = ((D > Dv ? D : Dv) + 63) / 64 * 64;
+  const size_t lds = ((size_t)D * Dv + 3 * (size_t)D + 16) * sizeof(float);
+  if (threads > 512 || lds > 160 * 1024 - 512) return MI_EUNSUPPORTED;
+  if (lds > 48 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(channel_delta_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return MI_ERUNTIME;
+  }
+  hipLaunchKernelGGL(channel_delta_kernel, dim3(n_seqs, H), dim3(threads), lds, S(stream), qkv, ld, q_off, k_off, v_off,
+                     beta_pre, ld_beta, decay_pre, ld_decay, dt_bias, a_log, gate_pre, ld_gate, norm_w, state, cu_q,
+                     kv_lens, slot_ids, H, G, D, Dv, eps, out, ldo);
+  return check_launch();
+}
+
+extern "C" int mi_route_grouped(const float* logits, int64_t ld, const float* correction, int n_tokens, int n_outputs,
+                                int top_k, int n_groups, int keep, int32_t* ids, float* weights, mi_stream stream) {
+  if (!logits || !correction || !ids || !weights || n_tokens < 0) return MI_EINVAL;
+  if (n_outputs < 1 || n_outputs > 512 || n_groups < 1 || n_outputs % n_groups || keep < 1 || keep > n_groups ||
+      top_k < 1 || top_k > keep * (n_outputs / n_groups))
+    return MI_EUNSUPPORTED;
+  if (n_tokens == 0) return MI_OK;
+  hipLaunchKernelGGL(route_grouped_kernel, dim3((n_tokens + 63) / 64), dim3(64), 0, S(stream), logits, ld, correction,
+                     n_tokens, n_outputs, top_k, n_groups, keep, ids, weights);
+  return check_launch();
+}
+
+extern "C" int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, const int32_t* ids, const float* weights,
+                                  int n_tokens, int top_k, int n_experts, int width, float* out, int64_t ldo,
+                                  mi_stream stream) {
+  if (!y || !h || !ids || !weights || !out || n_tokens < 0 || top_k < 1 || width < 1) return MI_EINVAL;
+  if (n_tokens == 0) return MI_OK;
+  hipLaunchKernelGGL(moe_combine_f32_kernel, dim3(n_tokens), dim3(256), 0, S(stream), y, h, ldh, ids, weights, top_k,
+                     n_experts, width, out, ldo);
+  return check_launch();
+}

@@ -24,6 +24,7 @@ LIB_PATH = os.environ.get(
 
 MI_OK = 0
 MI_EUNSUPPORTED = -2
+DTYPE_BF16, DTYPE_F32 = 0, 1
 HEAD_DIM = 128
 KV_TILE_TOKENS = 16
 KV_TILE_ELEMS = 2048
@@ -163,6 +164,21 @@ _SIGNATURES = {
     "mi_comm_set_spin_limit": (c_int, [_p, ctypes.c_uint32]),
     "mi_comm_status": (c_int, [_p, ctypes.POINTER(c_int)]),
     "mi_comm_timeout_info": (c_int, [_p, _p]),
+    "mi_gemm_any": (c_int, [_p, c_int64, _p, c_int, _p, c_int64, c_int, c_int, c_int, c_float, c_int, _p]),
+    "mi_gemm_any_grouped": (c_int, [_p, c_int64, _p, _p, _p, c_int, _p, c_int, c_int, _p, c_int64, _p, c_int, c_int,
+                                    c_int, _p]),
+    "mi_embedding_f32": (c_int, [_p, _p, c_int, _p, c_int, c_int, c_int, _p]),
+    "mi_layernorm_f32": (c_int, [_p, c_int64, _p, _p, _p, c_int64, c_int, c_int, c_float, c_int, _p]),
+    "mi_swa_prepare": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, _p, c_float, _p, c_int64, _p, _p, _p, c_int, _p,
+                               c_int, c_int, c_int, c_int, c_int, c_int, _p]),
+    "mi_swa_attention": (c_int, [_p, c_int64, _p, _p, c_int, _p, c_int, _p, _p, c_int, c_int, c_int, c_int, c_int,
+                                 c_int, c_int, c_int, c_float, _p, c_int64, _p, c_int64, _p]),
+    "mi_causal_conv_silu": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p]),
+    "mi_causal_conv_state": (c_int, [_p, c_int64, c_int, _p, _p, _p, _p, c_int, c_int, _p]),
+    "mi_channel_delta": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, c_int64, _p, c_int64, _p, _p, _p, c_int64, _p,
+                                 _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_int64, _p]),
+    "mi_route_grouped": (c_int, [_p, c_int64, _p, c_int, c_int, c_int, c_int, c_int, _p, _p, _p]),
+    "mi_moe_combine_f32": (c_int, [_p, _p, c_int64, _p, _p, c_int, c_int, c_int, c_int, _p, c_int64, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -54,6 +54,11 @@ class Config:
     # a prefill step at least this many tokens long has the next one queued behind it (engine/llm_engine.py); < 0: derived
     # after warm-up from this host's launch time and this device's time per token
     prefill_lookahead_min_tokens: int = -1
+    # serving dtype of the models that have an exact mode (32-bit-residual families): "bfloat16" | "float32"
+    dtype: str = "bfloat16"
+    # recurrent-state slots (models whose sequences carry a state beside their K/V pages); 0: max_num_seqs
+    num_state_slots: int = 0
+    hybrid_state: bool = False  # derived: the model class keeps recurrent state per sequence (no prefix sharing)
 
     def __post_init__(self):
         assert os.path.isdir(self.model), f"model must be a directory with a HF config.json: {self.model}"
@@ -63,10 +68,20 @@ class Config:
         assert self.quantization in (None, "fp8"), self.quantization
         if self.sampling_seed is None:
             self.sampling_seed = int.from_bytes(os.urandom(8), "little") >> 1
+        assert self.dtype in ("bfloat16", "float32"), self.dtype
+        if self.hf_config is None:
+            from nanovllm.models.models_map import native_config
+
+            self.hf_config = native_config(self.model, self.dtype)
         if self.hf_config is None:
             from transformers import AutoConfig
 
             self.hf_config = AutoConfig.from_pretrained(self.model, trust_remote_code=self.trust_remote_code)
+        if getattr(self.hf_config, "native", False):
+            from nanovllm.models.models_map import model_dict
+
+            self.hybrid_state = bool(getattr(model_dict[self.hf_config.architectures[0]], "hybrid_state", False))
+            self.hf_config.torch_dtype = self.dtype
         text = getattr(self.hf_config, "text_config", self.hf_config)
         max_pos = getattr(text, "max_position_embeddings", None)
         if max_pos is not None:

@@ -209,3 +209,61 @@ class BlockManager:
         h = self.compute_hash(toks, prev)
         tail.update(h, toks)
         self.hash_to_block_id[h] = tail.block_id
+
+
+class PlainBlockManager(BlockManager):
+    """Pages without prefix sharing, for models whose sequences also carry a recurrent state: a cache hit would bring
+    the K/V rows of a prefix back but not the state behind it, so every sequence owns its pages and nothing is hashed.
+    Same free-list discipline as BlockManager (FIFO, released last-block-first).  `extend` grows a table to cover a
+    sequence that is fed in portions."""
+
+    def allocate(self, seq: Sequence) -> None:
+        assert not seq.block_table
+        seq.table_gen = getattr(seq, "table_gen", 0) + 1
+        seq.num_prefix_tokens = 0
+        self.extend(seq, len(seq))
+
+    def can_extend(self, seq: Sequence, n_tokens: int) -> bool:
+        return len(self.free_block_ids) >= -(-n_tokens // self.block_size) - len(seq.block_table)
+
+    def extend(self, seq: Sequence, n_tokens: int) -> None:
+        need = -(-n_tokens // self.block_size) - len(seq.block_table)
+        if need > len(self.free_block_ids):
+            raise RuntimeError(f"out of KV pages: {need} needed, {len(self.free_block_ids)} free")
+        for _ in range(max(need, 0)):
+            bid = self.free_block_ids.popleft()
+            blk = self.blocks[bid]
+            assert blk.ref_count == 0
+            blk.reset()
+            self.used_block_ids.add(bid)
+            seq.block_table.append(bid)
+
+    def may_append(self, seq: Sequence, defer_seal: bool = False) -> bool:
+        self.extend(seq, len(seq))
+        return False
+
+    def seal_tail(self, seq: Sequence) -> None:
+        pass
+
+
+class StateSlots:
+    """Recurrent-state slots: one per live sequence of a hybrid model, handed out lowest-free-first and taken back when
+    the sequence ends or is preempted.  A slot is not cleared when it changes hands: the kernels start a sequence whose
+    first row is at position 0 from a zero state."""
+
+    def __init__(self, n_slots: int):
+        self.n_slots = n_slots
+        self.free = list(range(n_slots - 1, -1, -1))
+
+    def acquire(self, seq: Sequence) -> int:
+        if seq.state_slot < 0:
+            if not self.free:
+                raise RuntimeError(f"out of state slots ({self.n_slots})")
+            seq.state_slot = self.free.pop()
+        return seq.state_slot
+
+    def release(self, seq: Sequence) -> None:
+        if seq.state_slot >= 0:
+            self.free.append(seq.state_slot)
+            self.free.sort(reverse=True)
+            seq.state_slot = -1

@@ -27,6 +27,7 @@ import torch.distributed as dist
 from nanovllm import ops
 from nanovllm.config import Config
 from nanovllm.engine import batch_meta
+from nanovllm.engine.row_steps import RowSteps
 from nanovllm.engine.rpc import StepChannel
 from nanovllm.engine.sequence import Sequence
 from nanovllm.layers.sampler import Sampler
@@ -74,7 +75,7 @@ def graph_buckets(max_num_seqs: int) -> list[int]:
     return out
 
 
-class ModelRunner:
+class ModelRunner(RowSteps):
     def __init__(self, config: Config, rank: int, event=None):
         self.config = config
         self.hf_config = config.hf_config
@@ -139,9 +140,20 @@ class ModelRunner:
             self.xgmi_selftest = xgmi_comm.LAST_STATUS
 
         dtype = _torch_dtype_of(self.hf_config)
-        if dtype != torch.bfloat16:
+        arch = self.hf_config.architectures[0] if getattr(self.hf_config, "architectures", None) else "Qwen3ForCausalLM"
+        # hybrid models (recurrent-state slots beside the K/V pages, fp32 residual): the row-step path of
+        # engine/row_steps.py - eager launches, one GPU, bf16 or true fp32 weights and caches
+        self.hybrid = bool(getattr(model_dict[arch], "hybrid_state", False))
+        self.dtype = dtype
+        if self.hybrid:
+            if self.world_size > 1:
+                raise NotImplementedError(f"{arch}: tensor parallelism is not built for the hybrid-state models")
+            if dtype not in (torch.bfloat16, torch.float32):
+                raise NotImplementedError(f"{arch}: serving dtype {dtype}")
+        elif dtype != torch.bfloat16:
             raise NotImplementedError(f"the gfx950 kernels are bf16; checkpoint dtype is {dtype}")
-        self._check_supported_shapes()
+        if not self.hybrid:
+            self._check_supported_shapes()
         from nanovllm.layers.linear import set_weight_quantization
 
         set_weight_quantization(config.quantization)
@@ -149,8 +161,6 @@ class ModelRunner:
         torch.set_default_dtype(dtype)
         try:
             with torch.device(self.device):
-                arch = self.hf_config.architectures[0] if getattr(self.hf_config, "architectures", None) \
-                    else "Qwen3ForCausalLM"
                 self.model = model_dict[arch](self.hf_config)
         finally:
             torch.set_default_dtype(prev)
@@ -180,9 +190,17 @@ class ModelRunner:
         self.gather_logits = os.environ.get("MI355_TP_GATHER_LOGITS", "0") != "0"
         self._xgmi_flag = torch.zeros(1, dtype=torch.int32).pin_memory() if self.world_size > 1 else None
         torch.cuda.empty_cache()
+        self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        self.prefill_graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
+        if self.hybrid:  # pages + state slots, row staging; every step is launched eagerly
+            self.allocate_hybrid_cache()
+            self._alloc_row_staging()
+            self.graph_samples, self.graph_logits, self.prefill_graph_logits = set(), {}, {}
+            self.tokens_dev = torch.zeros(config.max_num_seqs, dtype=torch.int64, device=self.device)
+            self.prefill_graph_replays = 0
+            return
         self.allocate_kv_cache()
         self._alloc_staging()
-        self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.graph_samples: set[int] = set()  # buckets whose graph ends in the token choice, not in the logits
         self.graph_logits: dict[int, torch.Tensor] = {}
         # with TP the captured graph holds the xGMI exchange kernels; without them (RCCL all-reduce inside)
@@ -827,6 +845,8 @@ class ModelRunner:
     def run(self, seqs: list[Sequence], is_prefill: bool) -> list[int] | None:
         if not seqs:  # everything got preempted this step (reference would crash)
             return []
+        if self.hybrid:
+            return self.run_hybrid(seqs, is_prefill)
         real = len(seqs)
         if is_prefill and self.prefill_graphs:
             bucket = self._prefill_bucket(seqs, note=True)
@@ -903,7 +923,7 @@ class ModelRunner:
         a process group only: the TP workers' prefill ends in the exchange-status check of run(), and a step that issues
         RCCL collectives (also the one-rank group of MI355_TP1_COLLECTIVES) is waited for with the stream
         synchronisation of run()."""
-        return self.world_size == 1 and not self.collective
+        return self.world_size == 1 and not self.collective and not self.hybrid
 
     def prefill_launchable(self, seqs: list[Sequence]) -> bool:
         """May THIS prefill step be queued without waiting for its tokens?  One GPU: any step (eagerly if it has no

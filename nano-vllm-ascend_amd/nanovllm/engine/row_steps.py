@@ -1,0 +1,131 @@
+"""The step function of hybrid models (sequences that own recurrent-state slots beside their K/V pages).
+
+A step is a list of ROW RUNS, one per sequence: `count` tokens that continue the sequence at position `start` - a whole
+prompt, a portion of one, or a single decoded token; the kernels make no difference between them (layers/seqmix.py), so
+portions of prompts and decoded tokens of other sequences share a batch.  ModelRunner mixes this class in: `run()` turns
+the scheduler's prefill / decode steps into row runs, a trace replay (bin/trace_run) calls `run_rows` with the cut it was
+given.
+
+Metadata reaches the device as in ModelRunner.prepare_prefill: every array of the step packed into one pinned staging
+buffer (two, alternating) and uploaded with one copy.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from nanovllm.utils.context import reset_context, set_context
+
+
+class RowSteps:
+    # ------------------------------------------------------------------ cache and state
+    def allocate_hybrid_cache(self):
+        """Pages for the attention layers and state slots for the recurrent ones.  num_kvcache_blocks counts the reserved
+        last block as in the paged-attention models' cache (the scheduler hands out the others)."""
+        cfg = self.config
+        item = 4 if self.dtype == torch.float32 else 2
+        per_block = max(1, self.model.cache_bytes_per_block(self.block_size, item))
+        n_slots = cfg.num_state_slots or cfg.max_num_seqs
+        if cfg.num_kvcache_blocks <= 0:
+            free, total = torch.cuda.mem_get_info(self.device)
+            budget = total * cfg.gpu_memory_utilization - (total - free) - n_slots * self.model.state_bytes_per_slot()
+            cfg.num_kvcache_blocks = int(budget) // per_block
+        assert cfg.num_kvcache_blocks > 1, "no memory left for the K/V pages"
+        self.n_state_slots = n_slots
+        self.model.bind_cache(cfg.num_kvcache_blocks, self.block_size, n_slots, self.dtype, self.device)
+
+    def _alloc_row_staging(self):
+        nbytes = 1 << 16
+        self._row_hosts = [torch.empty(nbytes, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
+        self._row_dev = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        self._row_flip = 0
+        self._row_events = [None, None]
+
+    # ------------------------------------------------------------------ metadata
+    def prepare_rows(self, runs, want):
+        """runs: [(sequence, start, count)], want: step rows whose logits are asked for.  Installs the step's context and
+        returns (input ids, wanted rows) on the device."""
+        bs = self.block_size
+        n = len(runs)
+        counts = np.fromiter((c for _, _, c in runs), dtype=np.int64, count=n)
+        cu = np.zeros(n + 1, dtype=np.int32)
+        np.cumsum(counts, out=cu[1:])
+        total = int(cu[-1])
+        ids = np.empty(total, dtype=np.int64)
+        slots = np.empty(total, dtype=np.int32)
+        kv_lens = np.empty(n, dtype=np.int32)
+        state_slots = np.empty(n, dtype=np.int32)
+        width = max(1, max(-(-(s0 + c) // bs) for _, s0, c in runs))
+        tables = np.full((n, width), -1, dtype=np.int32)
+        for i, (seq, start, count) in enumerate(runs):
+            a = int(cu[i])
+            assert count >= 1 and start + count <= len(seq) and len(seq.block_table) * bs >= start + count, \
+                (start, count, len(seq), len(seq.block_table))
+            ids[a:a + count] = seq.token_ids[start:start + count]
+            pos = np.arange(start, start + count)
+            table = np.asarray(seq.block_table, dtype=np.int32)
+            slots[a:a + count] = table[pos // bs] * bs + pos % bs
+            kv_lens[i] = start + count
+            assert seq.state_slot >= 0
+            state_slots[i] = seq.state_slot
+            nb = -(-(start + count) // bs)
+            tables[i, :nb] = table[:nb]
+        want = np.asarray(want, dtype=np.int64)
+        arrays = (ids, slots, cu, kv_lens, state_slots, tables, want)
+        offs, off = [], 0
+        for a in arrays:
+            offs.append(off)
+            off += (a.nbytes + 15) // 16 * 16
+        self._row_flip ^= 1
+        b = self._row_flip
+        if self._row_events[b] is not None:
+            self._row_events[b].synchronize()  # the upload that last read this pinned buffer has run
+        if off > self._row_hosts[b].numel():
+            self._row_hosts[b] = torch.empty(off * 2, dtype=torch.uint8, pin_memory=True)
+        if off > self._row_dev.numel():
+            self._row_dev = torch.empty(off * 2, dtype=torch.uint8, device=self.device)
+        host = self._row_hosts[b].numpy()
+        for a, o in zip(arrays, offs):
+            host[o:o + a.nbytes] = np.ascontiguousarray(a).reshape(-1).view(np.uint8)
+        self._row_dev[:off].copy_(self._row_hosts[b][:off], non_blocking=True)
+        ev = self._row_events[b] or torch.cuda.Event()
+        ev.record()
+        self._row_events[b] = ev
+
+        def dev(i, dtype, shape=None):
+            t = self._row_dev[offs[i]:offs[i] + arrays[i].nbytes].view(dtype)
+            return t if shape is None else t.view(shape)
+
+        set_context(True, cu_seqlens_q=dev(2, torch.int32), kv_lens=dev(3, torch.int32), slot_mapping=dev(1, torch.int32),
+                    block_tables=dev(5, torch.int32, tables.shape), block_size=bs, state_slots=dev(4, torch.int32),
+                    max_seqlen_q=int(counts.max()), max_seqlen_k=int(kv_lens.max()))
+        return dev(0, torch.int64), dev(6, torch.int64)
+
+    # ------------------------------------------------------------------ one step
+    @torch.inference_mode()
+    def run_rows(self, runs, want=None) -> torch.Tensor:
+        """One step over the row runs; returns fp32 logits [len(want), vocab] on the device (default: each run's last row).
+        The sequences' pages and state slots must be in place (Scheduler.admit_portion / schedule())."""
+        if want is None:
+            ends = np.cumsum([c for _, _, c in runs])
+            want = (ends - 1).tolist()
+        input_ids, rows = self.prepare_rows(runs, want)
+        hidden = self.model(input_ids)
+        logits = self.model.compute_logits(hidden, rows) if len(want) else None
+        for seq, start, count in runs:
+            seq.num_computed_tokens = start + count
+        self._steps_run += 1
+        reset_context()
+        return logits
+
+    def run_hybrid(self, seqs, is_prefill: bool) -> list[int]:
+        """ModelRunner.run for a hybrid model: the scheduler's prefill step (whole prompts; a preempted sequence comes back
+        with its completion tokens and is recomputed from position 0, its state from zero) or decode step as row runs,
+        then the framework's sampler on the last rows."""
+        runs = [(s, 0, len(s)) if is_prefill else (s, len(s) - 1, 1) for s in seqs]
+        logits = self.run_rows(runs)
+        self.last_logits = logits
+        real = len(seqs)
+        temps = torch.tensor([0.0 if s.greedy else s.temperature for s in seqs], dtype=torch.float32).to(self.device)
+        self.sampler(logits.to(torch.bfloat16), temps, out=self.tokens_dev[:real])
+        return self.tokens_dev[:real].tolist()

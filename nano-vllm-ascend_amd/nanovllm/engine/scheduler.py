@@ -11,7 +11,7 @@ from __future__ import annotations
 
 from collections import deque
 
-from nanovllm.engine.block_manager import BlockManager
+from nanovllm.engine.block_manager import BlockManager, PlainBlockManager, StateSlots
 from nanovllm.engine.sequence import FinishReason, Sequence, SequenceStatus
 
 
@@ -23,7 +23,11 @@ class Scheduler:
         self.eos = config.eos
         # the last KV block is reserved as the dummy slot of graph-padded rows
         # (scheduler.py:26-30, model_runner.py:309)
-        self.block_manager = BlockManager(config.num_kvcache_blocks - 1, config.kvcache_block_size)
+        # hybrid models (recurrent state beside the K/V pages): no prefix sharing, one state slot per live sequence
+        hybrid = bool(getattr(config, "hybrid_state", False))
+        self.block_manager = (PlainBlockManager if hybrid else BlockManager)(config.num_kvcache_blocks - 1,
+                                                                             config.kvcache_block_size)
+        self.state_slots = StateSlots(getattr(config, "num_state_slots", 0) or config.max_num_seqs) if hybrid else None
         self.waiting: deque[Sequence] = deque()
         self.running: deque[Sequence] = deque()
 
@@ -46,6 +50,11 @@ class Scheduler:
             seq = self.waiting[0]
             if budget_used + len(seq) > self.max_num_batched_tokens or not bm.can_allocate(seq):
                 break
+            if self.state_slots is not None:
+                if not self.state_slots.free:
+                    break
+                self.state_slots.acquire(seq)
+                seq.num_computed_tokens = 0
             self.waiting.popleft()
             bm.allocate(seq)
             seq.status = SequenceStatus.RUNNING
@@ -87,6 +96,8 @@ class Scheduler:
         seq.status = SequenceStatus.WAITING
         seq.finish_reason = FinishReason.PREEMPTED
         self.block_manager.deallocate(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
         self.waiting.appendleft(seq)
 
     # -- request lifecycle -------------------------------------------------------------------------
@@ -100,6 +111,29 @@ class Scheduler:
         seq.status = SequenceStatus.FINISHED
         seq.finish_reason = reason
         self.block_manager.deallocate(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
+
+    # -- sequences fed in portions (a replayed trace dictates the cut; hybrid models) ---------------------------
+    def admit_portion(self, seq: Sequence, token_ids: list[int]) -> None:
+        """The next tokens of `seq` are about to be computed in one step beside other sequences' rows: a new sequence
+        joins `running` and gets its state slot, its table grows to cover the tokens."""
+        assert self.state_slots is not None, "portion-wise feeding is the hybrid models' row-step path"
+        if seq.status is not SequenceStatus.RUNNING:
+            if len(self.running) >= self.max_num_seqs:
+                raise RuntimeError(f"more than max_num_seqs = {self.max_num_seqs} live sequences")
+            seq.status = SequenceStatus.RUNNING
+            seq.table_gen += 1
+            self.running.append(seq)
+        self.state_slots.acquire(seq)
+        seq.extend_tokens(token_ids)
+        self.block_manager.extend(seq, len(seq))
+
+    def finish(self, seq: Sequence) -> None:
+        """A sequence fed in portions is over: pages and slot go back."""
+        self.free_seq(seq, FinishReason.LENGTH)
+        if seq in self.running:
+            self.running.remove(seq)
 
     # -- lookahead: schedule step k+1 while step k's tokens are still on the device -------------------
     def _ends_by_length(self, seq: Sequence) -> bool:

@@ -32,7 +32,7 @@ class Sequence:
     __slots__ = ("block_size", "seq_id", "request_id", "status", "token_ids", "last_token", "num_tokens",
                  "num_prompt_tokens", "num_cached_tokens", "block_table", "temperature", "max_tokens",
                  "ignore_eos", "greedy", "finish_reason", "arrival_time", "first_token_time", "table_gen", "num_prefix_tokens",
-                 "token_pending", "_prompt_q", "_prompt_hashes")
+                 "token_pending", "_prompt_q", "_prompt_hashes", "state_slot", "num_computed_tokens")
 
     def __init__(self, token_ids: list[int], sampling_params: SamplingParams | None = None,
                  request_id: str | None = None, block_size: int = 256, **_ignored_multimodal):
@@ -56,6 +56,8 @@ class Sequence:
         self.num_prefix_tokens = 0  # leading tokens whose KV rows the current block table already holds (cache hits)
         self.token_pending = False  # the last entry of token_ids stands for a token still on the device (lookahead)
         self.table_gen = 0  # bumped every time the block table is rebuilt (allocate after a preemption)
+        self.state_slot = -1  # recurrent-state slot (hybrid models; engine/block_manager.py: StateSlots)
+        self.num_computed_tokens = 0  # row-step engines: tokens whose K/V rows and state are in place (prompt portions)
         # Request preprocessing, done when the request is CREATED (like tokenisation; the reference's serving bench starts
         # a request's clock after add_request has returned, bench/serving_bench.py:100-105): the prompt as array('q')
         # (block hashing and the prefill staging read it: ~20 us per 1024 tokens) and, on first allocation, the chained
@@ -138,6 +140,14 @@ class Sequence:
         self.last_token = token_id
         self.num_tokens += 1
 
+    def extend_tokens(self, token_ids: list[int]) -> None:
+        """More tokens of a sequence that is fed in portions (a replayed trace names them step by step)."""
+        if token_ids:
+            self.token_ids.extend(token_ids)
+            self.last_token = self.token_ids[-1]
+            self.num_tokens += len(token_ids)
+            self._prompt_q = None
+
     def append_pending(self) -> None:
         """Count a token that has been sampled on the device but has not reached the host (engine lookahead)."""
         assert not self.token_pending
@@ -194,4 +204,5 @@ class Sequence:
         s.max_tokens, s.ignore_eos, s.finish_reason = 0, True, None
         s.arrival_time = s.first_token_time = 0.0
         s.token_pending = False
+        s.state_slot, s.num_computed_tokens = -1, 0
         return s, pos

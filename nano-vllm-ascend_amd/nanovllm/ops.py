@@ -929,3 +929,183 @@ def add_rmsnorm_splitk_stamped(partials, residual, w, eps: float, stamps, out=No
     check(lib.mi_add_rmsnorm_splitk_ex(ptr(partials), nsplit, ptr(residual), ptr(w), ptr(out), ptr(residual_out), rows,
                                        cols, float(eps), ptr(stamps), stream()), "mi_add_rmsnorm_splitk_ex")
     return out, residual_out
+
+
+# --------------------------------------------------------------------------- 32-bit-residual model families
+# (csrc/gemm_any.hip, csrc/seqmix.hip).  Activations are fp32 tensors; weights, tables and K/V caches are bf16 or fp32.
+_F32 = torch.float32
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == _BF16:
+        return _C.DTYPE_BF16
+    if t.dtype == _F32:
+        return _C.DTYPE_F32
+    raise _C.MiError(f"expected a bfloat16 or float32 tensor, got {t.dtype}")
+
+
+def _f32(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is not None and (t.dtype != _F32 or t.stride(-1) != 1):
+            raise _C.MiError(f"expected a float32 tensor with unit inner stride, got {t.dtype} / strides {t.stride()}")
+
+
+def _i32(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()):
+            raise _C.MiError("expected a contiguous int32 tensor")
+
+
+def gemm_any(x, w, alpha: float = 1.0, exact: bool = False, out=None) -> torch.Tensor:
+    """alpha * x @ w.T for any shapes; x may be a column slice of a wider buffer (unit inner stride)."""
+    require_gpu(x, w)
+    _f32(x, out)
+    assert x.dim() == 2 and w.dim() == 2 and w.is_contiguous() and x.shape[1] == w.shape[1], (x.shape, w.shape)
+    M, K = x.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=_F32, device=x.device)
+    assert out.shape == (M, N)
+    check(lib.mi_gemm_any(ptr(x), x.stride(0) if M > 1 else K, ptr(w), _dt(w), ptr(out), out.stride(0) if M > 1 else N,
+                          M, N, K, float(alpha), int(exact), stream()), "mi_gemm_any")
+    return out
+
+
+def gemm_any_grouped(x, x_rows, w, w2, group_offsets, rows_max: int, y_rows, y_rows_total: int, exact: bool = False):
+    """Per group g (an expert): y[rows of g] = x[rows of g] @ w[g].T, or silu(x w[g].T) * (x w2[g].T) with w2."""
+    require_gpu(x, w, group_offsets)
+    _f32(x)
+    _i32(x_rows, y_rows, group_offsets)
+    assert w.dim() == 3 and w.is_contiguous() and (w2 is None or (w2.shape == w.shape and w2.is_contiguous() and w2.dtype == w.dtype))
+    G, N, K = w.shape
+    assert x.shape[1] == K and group_offsets.numel() >= G + 1
+    y = torch.empty((y_rows_total, N), dtype=_F32, device=x.device)
+    check(lib.mi_gemm_any_grouped(ptr(x), x.stride(0), ptr(x_rows), ptr(w), ptr(w2), _dt(w), ptr(group_offsets), G,
+                                  rows_max, ptr(y), N, ptr(y_rows), N, K, int(exact), stream()), "mi_gemm_any_grouped")
+    return y
+
+
+def embedding_f32(ids, table) -> torch.Tensor:
+    require_gpu(ids, table)
+    assert ids.dtype == torch.int64 and ids.is_contiguous() and table.is_contiguous()
+    out = torch.empty((ids.numel(), table.shape[1]), dtype=_F32, device=table.device)
+    check(lib.mi_embedding_f32(ptr(ids), ptr(table), _dt(table), ptr(out), ids.numel(), table.shape[1], table.shape[0],
+                               stream()), "mi_embedding_f32")
+    return out
+
+
+def layernorm_f32(y, w, b, eps: float, add_to=None) -> torch.Tensor:
+    """LN(y) * w + b per row; add_to: the residual it is added to IN PLACE (returned)."""
+    require_gpu(y, w, b)
+    _f32(y, w, b, add_to)
+    rows, width = y.shape
+    out = add_to if add_to is not None else torch.empty((rows, width), dtype=_F32, device=y.device)
+    assert out.shape == y.shape and w.numel() == width and b.numel() == width
+    check(lib.mi_layernorm_f32(ptr(y), y.stride(0), ptr(w), ptr(b), ptr(out), out.stride(0), rows, width, float(eps),
+                               int(add_to is not None), stream()), "mi_layernorm_f32")
+    return out
+
+
+def swa_prepare(proj, q_off: int, k_off: int, v_off: int, qn_w, kn_w, eps: float, v_first, lam, k_cache, v_cache,
+                slots, H: int, G: int, D: int, Dv: int, block_size: int) -> None:
+    require_gpu(proj, k_cache, v_cache, slots)
+    _f32(proj, qn_w, kn_w, v_first, lam)
+    _i32(slots)
+    rows = proj.shape[0]
+    assert slots.numel() == rows and qn_w.numel() == H * D and kn_w.numel() == G * D and k_cache.dtype == v_cache.dtype
+    assert k_cache.shape[1:] == (G, block_size, D) and v_cache.shape[1:] == (G, block_size, Dv), (k_cache.shape, v_cache.shape)
+    assert max(q_off + H * D, k_off + G * D, v_off + G * Dv) <= proj.shape[1]
+    assert v_first is None or (v_first.shape[0] == rows and v_first.shape[1] >= G * Dv and lam is not None)
+    check(lib.mi_swa_prepare(ptr(proj), proj.stride(0), q_off, k_off, v_off, ptr(qn_w), ptr(kn_w), float(eps),
+                             ptr(v_first), v_first.stride(0) if v_first is not None else 0, ptr(lam), ptr(k_cache),
+                             ptr(v_cache), _dt(k_cache), ptr(slots), rows, H, G, D, Dv, block_size, stream()),
+          "mi_swa_prepare")
+
+
+def swa_attention(q, k_cache, v_cache, block_tables, cu_q, kv_lens, H: int, G: int, D: int, Dv: int, block_size: int,
+                  window: int, scale: float, gate=None) -> torch.Tensor:
+    require_gpu(q, k_cache, v_cache, block_tables, cu_q, kv_lens)
+    _f32(q, gate)
+    _i32(block_tables, cu_q, kv_lens)
+    rows, n_seqs = q.shape[0], kv_lens.numel()
+    assert q.shape[1] >= H * D and cu_q.numel() == n_seqs + 1 and block_tables.shape[0] >= n_seqs
+    out = torch.empty((rows, H * Dv), dtype=_F32, device=q.device)
+    check(lib.mi_swa_attention(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), _dt(k_cache), ptr(block_tables),
+                               block_tables.shape[1], ptr(cu_q), ptr(kv_lens), n_seqs, rows, H, G, D, Dv, block_size,
+                               int(window), float(scale), ptr(gate), gate.stride(0) if gate is not None else 0,
+                               ptr(out), out.stride(0), stream()), "mi_swa_attention")
+    return out
+
+
+def causal_conv_silu(x, w, state, cu_q, kv_lens, slot_ids) -> torch.Tensor:
+    """silu(depthwise causal conv); `state` [slots, taps - 1, C] is READ here and advanced by causal_conv_state()."""
+    require_gpu(x, w, state)
+    _f32(x, w, state)
+    _i32(cu_q, kv_lens, slot_ids)
+    rows, C = x.shape
+    taps = w.shape[1]
+    assert w.shape[0] == C and w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (max(taps - 1, 0), C)
+    y = torch.empty((rows, C), dtype=_F32, device=x.device)
+    check(lib.mi_causal_conv_silu(ptr(x), x.stride(0), ptr(w), taps, ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
+                                  kv_lens.numel(), rows, C, ptr(y), C, stream()), "mi_causal_conv_silu")
+    return y
+
+
+def causal_conv_state(x, taps: int, state, cu_q, kv_lens, slot_ids) -> None:
+    require_gpu(x, state)
+    _f32(x, state)
+    check(lib.mi_causal_conv_state(ptr(x), x.stride(0), taps, ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
+                                   kv_lens.numel(), x.shape[1], stream()), "mi_causal_conv_state")
+
+
+def channel_delta(qkv, q_off: int, k_off: int, v_off: int, beta_pre, decay_pre, dt_bias, a_log, gate_pre, norm_w, state,
+                  cu_q, kv_lens, slot_ids, H: int, G: int, D: int, Dv: int, eps: float) -> torch.Tensor:
+    require_gpu(qkv, state)
+    _f32(qkv, beta_pre, decay_pre, dt_bias, a_log, gate_pre, norm_w, state)
+    _i32(cu_q, kv_lens, slot_ids)
+    rows = qkv.shape[0]
+    assert state.is_contiguous() and state.shape[1:] == (H, D, Dv), state.shape
+    assert beta_pre.shape == (rows, H) and decay_pre.shape == (rows, H * D) and gate_pre.shape == (rows, H * Dv)
+    assert dt_bias.numel() == H * D and a_log.numel() == H and norm_w.numel() == Dv
+    out = torch.empty((rows, H * Dv), dtype=_F32, device=qkv.device)
+    check(lib.mi_channel_delta(ptr(qkv), qkv.stride(0), q_off, k_off, v_off, ptr(beta_pre), beta_pre.stride(0),
+                               ptr(decay_pre), decay_pre.stride(0), ptr(dt_bias), ptr(a_log), ptr(gate_pre),
+                               gate_pre.stride(0), ptr(norm_w), ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
+                               kv_lens.numel(), H, G, D, Dv, float(eps), ptr(out), out.stride(0), stream()),
+          "mi_channel_delta")
+    return out
+
+
+def route_grouped(logits, correction, top_k: int, n_groups: int, keep: int):
+    require_gpu(logits, correction)
+    _f32(logits, correction)
+    T, n = logits.shape
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    wts = torch.empty((T, top_k), dtype=_F32, device=logits.device)
+    check(lib.mi_route_grouped(ptr(logits), logits.stride(0), ptr(correction), T, n, top_k, n_groups, keep, ptr(ids),
+                               ptr(wts), stream()), "mi_route_grouped")
+    return ids, wts
+
+
+def moe_sort(ids, n_outputs: int):
+    """(offsets [n_outputs + 1], pair_token [P], pair_index [P]) of the (token, slot) pairs grouped by router output."""
+    T, top_k = ids.shape
+    dev = ids.device
+    offsets = torch.empty(n_outputs + 1, dtype=torch.int32, device=dev)
+    pair_token = torch.empty(T * top_k, dtype=torch.int32, device=dev)
+    pair_index = torch.empty(T * top_k, dtype=torch.int32, device=dev)
+    check(lib.mi_moe_sort(ptr(ids), T, top_k, n_outputs, ptr(offsets), ptr(pair_token), ptr(pair_index), stream()),
+          "mi_moe_sort")
+    return offsets, pair_token, pair_index
+
+
+def moe_combine_f32(y, h, ids, wts, n_experts: int) -> torch.Tensor:
+    require_gpu(y, h, ids, wts)
+    _f32(y, h, wts)
+    T, top_k = ids.shape
+    width = h.shape[1]
+    assert y.shape == (T * top_k, width) and y.is_contiguous()
+    out = torch.empty((T, width), dtype=_F32, device=h.device)
+    check(lib.mi_moe_combine_f32(ptr(y), ptr(h), h.stride(0), ptr(ids), ptr(wts), T, top_k, n_experts, width, ptr(out),
+                                 width, stream()), "mi_moe_combine_f32")
+    return out

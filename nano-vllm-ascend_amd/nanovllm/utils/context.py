@@ -32,6 +32,7 @@ _DEFAULTS = {
     "kv_lens": None,
     "token_src": None,         # int32 [B]: row of prev_tokens a decode row takes its input id from, or -1
     "prev_tokens": None,       # int64 [>= B]: the previous step's sampled tokens, device-resident
+    "state_slots": None,       # int32 [n_seqs]: recurrent-state slot of each sequence of the step (hybrid models)
 }
 
 

@@ -23,7 +23,11 @@ def has_checkpoint(path: str) -> bool:
     return bool(glob(os.path.join(path, "*.safetensors")))
 
 
-def _route(model: nn.Module, name: str, tensor: torch.Tensor) -> None:
+def _route(model: nn.Module, name, tensor: torch.Tensor) -> None:
+    if isinstance(name, tuple):  # (parameter, shard): a model's own name map (map_checkpoint_name) already resolved it
+        param = model.get_parameter(name[0])
+        param.weight_loader(param, tensor.to(param.dtype), name[1])
+        return
     mapping = getattr(model, "packed_modules_mapping", {})
     for src, (dst, shard_id) in mapping.items():
         if src in name:
@@ -52,6 +56,8 @@ def load_model(model: nn.Module, path: str, name_mapping=None) -> None:
     from safetensors import safe_open
 
     tied = getattr(getattr(model, "lm_head", None), "weight", None)
+    if name_mapping is None:  # a model whose checkpoint names are not its parameter paths brings its own map
+        name_mapping = getattr(model, "map_checkpoint_name", None)
     for file in sorted(glob(os.path.join(path, "*.safetensors"))):
         with safe_open(file, "pt", "cpu") as f:
             for name in f.keys():
@@ -121,6 +127,12 @@ def synthetic_state(hf_config, seed: int = 0, std: float = 0.02, dtype=torch.bfl
 
 
 def init_synthetic_weights(model: nn.Module, hf_config, seed: int = 0, std: float = 0.02) -> None:
+    own = getattr(model, "synthetic_state", None)  # a model that names its own random checkpoint
+    if own is not None:
+        for name, tensor in own(seed):
+            _route(model, model.map_checkpoint_name(name), tensor)
+        pack_model_weights(model)
+        return
     for name, tensor in synthetic_state(hf_config, seed, std):
         _route(model, name, tensor)
     pack_model_weights(model)
