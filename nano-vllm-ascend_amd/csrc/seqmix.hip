@@ -220,8 +220,8 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(const float* __re
                                                                const int32_t* __restrict__ kv_lens,
                                                                const int32_t* __restrict__ slot_ids, int n_seqs, int C,
                                                                float* __restrict__ y, int64_t ldy) {
-  const int row = blockIdx.y;
-  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int row = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int s = seq_of_row(cu_q, n_seqs, row);
   const int r = row - cu_q[s];
@@ -496,8 +496,7 @@ extern "C" int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, 
   if (!x || !w || !state || !cu_q || !kv_lens || !slot_ids || !y || rows < 0 || n_seqs < 1 || channels < 1) return MI_EINVAL;
   if (taps < 1 || taps > 17) return MI_EUNSUPPORTED;
   if (rows == 0) return MI_OK;
-  if (rows > 65535) return MI_EUNSUPPORTED;
-  hipLaunchKernelGGL(causal_conv_silu_kernel, dim3((channels + 255) / 256, rows), dim3(256), 0, S(stream), x, ldx, w,
+  hipLaunchKernelGGL(causal_conv_silu_kernel, dim3(rows, (channels + 255) / 256), dim3(256), 0, S(stream), x, ldx, w,
                      taps, state, cu_q, kv_lens, slot_ids, n_seqs, channels, y, ldy);
   return check_launch();
 }

@@ -116,7 +116,8 @@ class GazutarForCausalLM(nn.Module):
 
     # ---- checkpoint names -> parameters (utils/loader.py) ------------------------------------------------------
     def map_checkpoint_name(self, name: str):
-        """-> parameter path, or (parameter path, shard) for tensors that land inside a merged / stacked parameter."""
+        """-> parameter path, (parameter path, shard) for tensors that land inside a merged / stacked parameter, or None
+        for a tensor this configuration has no use for."""
         if name in ("embed", "head"):
             return name
         if name.startswith("final.norm"):
@@ -125,6 +126,8 @@ class GazutarForCausalLM(nn.Module):
         i = int(layer[1:])
         pre = f"layers.{i}."
         if rest.startswith("norm"):
+            if rest.startswith("norm2") and self.layers[i].mlp is None:
+                return None  # (a layer without feed-forward has no second norm: a tensor of that name is ignored)
             return pre + (rest[:-2] + ".bias" if rest.endswith(".b") else rest + ".weight")
         part, leaf = rest.split(".", 1)
         if part == "mlp":

@@ -1044,7 +1044,7 @@ def causal_conv_silu(x, w, state, cu_q, kv_lens, slot_ids) -> torch.Tensor:
     _i32(cu_q, kv_lens, slot_ids)
     rows, C = x.shape
     taps = w.shape[1]
-    assert w.shape[0] == C and w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (max(taps - 1, 0), C)
+    assert w.shape[0] == C and w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (max(taps - 1, 1), C)
     y = torch.empty((rows, C), dtype=_F32, device=x.device)
     check(lib.mi_causal_conv_silu(ptr(x), x.stride(0), ptr(w), taps, ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
                                   kv_lens.numel(), rows, C, ptr(y), C, stream()), "mi_causal_conv_silu")

@@ -50,6 +50,21 @@ def slopes(n_heads, dtype):
     return torch.tensor([2.0 ** (-8.0 * (h + 1) / n_heads) for h in range(n_heads)], dtype=dtype)
 
 
+def windowed_attention(q, k, v, scale, window):
+    """q [T, H, D], k [T, G, D], v [T, G, Dv] of one sequence -> [T, H, Dv]; dense scores, -inf outside the window."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    dist = torch.arange(T).view(T, 1) - torch.arange(T).view(1, T)
+    visible = (dist >= 0) & (dist < window)
+    sl = slopes(H, q.dtype)
+    out = torch.empty(T, H, v.shape[-1], dtype=q.dtype)
+    for hd in range(H):
+        g = hd // (H // G)
+        s = (q[:, hd] @ k[:, g].T) * scale - sl[hd] * dist.to(q.dtype)
+        out[:, hd] = torch.softmax(s.masked_fill(~visible, float("-inf")), -1) @ v[:, g]
+    return out
+
+
 def attention_mixer(h, p, cfg, eps, v_first, is_first_vmix):
     """h [T, W] of ONE sequence -> (mixer output [T, W], this layer's values as cached [T, G * vdim])."""
     T = h.shape[0]
@@ -60,18 +75,7 @@ def attention_mixer(h, p, cfg, eps, v_first, is_first_vmix):
     if cfg.get("v_mix") and not is_first_vmix:
         lam = p["vmix"]
         v = (1 - lam) * v + lam * v_first
-    vh = v.view(T, G, Dv)
-    i = torch.arange(T).view(T, 1)
-    j = torch.arange(T).view(1, T)
-    dist = (i - j)
-    visible = (dist >= 0) & (dist < cfg["mask"]["size"])
-    sl = slopes(H, h.dtype)
-    out = torch.empty(T, H, Dv, dtype=h.dtype)
-    for hd in range(H):
-        g = hd // (H // G)
-        s = (q[:, hd] @ k[:, g].T) * cfg["scale"] - sl[hd] * dist.to(h.dtype)
-        s = s.masked_fill(~visible, float("-inf"))
-        out[:, hd] = torch.softmax(s, -1) @ vh[:, g]
+    out = windowed_attention(q, k, v.view(T, G, Dv), cfg["scale"], cfg["mask"]["size"])
     gate = torch.sigmoid(h @ p["g"].T)
     return (out.reshape(T, H * Dv) * gate) @ p["o"].T, v
 
