@@ -127,5 +127,9 @@ class RowSteps:
         self.last_logits = logits
         real = len(seqs)
         temps = torch.tensor([0.0 if s.greedy else s.temperature for s in seqs], dtype=torch.float32).to(self.device)
-        self.sampler(logits.to(torch.bfloat16), temps, out=self.tokens_dev[:real])
+        # the sampler reads bf16 logits in rows of a multiple of 8 elements (layers/sampler.py)
+        vocab = logits.shape[1]
+        rounded = torch.empty((real, -(-vocab // 8) * 8), dtype=torch.bfloat16, device=self.device)[:, :vocab]
+        rounded.copy_(logits)
+        self.sampler(rounded, temps, out=self.tokens_dev[:real])
         return self.tokens_dev[:real].tolist()

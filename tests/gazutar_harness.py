@@ -54,10 +54,30 @@ def write_model_dir(cfg: dict, weights: dict) -> str:
     return d
 
 
-def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
-    """Largest row-wise rms difference relative to the rms of the expected logits."""
+def row_errs(got: torch.Tensor, want: torch.Tensor) -> torch.Tensor:
+    """Row-wise rms difference relative to the rms of the expected row."""
     got, want = got.double(), want.double()
-    return float(((got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt().clamp_min(1e-9)).max())
+    return (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    return float(row_errs(got, want).max())
+
+
+F32_BAR, BF16_BAR = 5e-5, 3e-2
+
+
+def assert_close(got: torch.Tensor, want: torch.Tensor, dtype: str, what="") -> None:
+    """float32 mode: every row within F32_BAR.  bfloat16 mode: rounding noise of a few 1e-3 per row - but a router's
+    near-tie that falls the other way under bf16 rounding replaces an expert for that token and moves its row (and,
+    through the recurrent state, every later row of the sequence) by tens of percent, so up to a quarter of the rows may be
+    off; position-exact faults are the float32 runs' business."""
+    e = row_errs(got, want)
+    if dtype == "float32":
+        assert float(e.max()) <= F32_BAR, (what, float(e.max()), int(e.argmax()))
+    else:
+        off = int((e > BF16_BAR).sum())
+        assert float(e.median()) <= BF16_BAR / 2 and off <= max(1, e.numel() // 4), (what, float(e.median()), off, e.numel())
 
 
 class Replay:
