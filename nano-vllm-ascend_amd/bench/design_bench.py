@@ -1,0 +1,123 @@
+"""Prefill and decode throughput of a model design beside the framework's closest existing model at equal size
+(`python bench.py --design gazutar`): random weights, layer sizes that resemble a real model's, both models through the same
+engine entry points (add_request / step), each served the way the framework serves it (Qwen3-MoE: captured prefill and
+decode steps; Gazutar: what ModelRunner reports in `served_as`).
+
+One JSON line: per size, per model: prefill tokens/s (all prompts, wall clock around the prefill steps), decode tokens/s and
+ms per decode step (wall clock around `steps` engine steps of the full batch), weight bytes a decode step streams and the
+fraction of the 8 TB/s HBM roofline that makes.
+"""
+from __future__ import annotations
+
+import json
+import random
+import time
+
+HBM_BYTES_PER_S = 8.0e12
+
+# (name, width, layers, heads, kv heads, head dim, experts, expert ff, top k, vocab, window)
+SIZES = {
+    "w1024": dict(width=1024, layers=4, heads=8, kv_heads=4, dim=128, experts=32, ff=512, top=4, vocab=32768, window=512),
+    "w2048": dict(width=2048, layers=4, heads=16, kv_heads=8, dim=128, experts=64, ff=768, top=8, vocab=32768, window=1024),
+}
+
+
+def gazutar_config(s: dict) -> dict:
+    att = {"type": "attention", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"],
+                                          "mask": {"size": s["window"]}, "scale": s["dim"] ** -0.5, "v_mix": True}}
+    rec = {"type": "channel_delta", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"],
+                                              "vdim": s["dim"], "conv": 4, "rank": s["width"] // 16}}
+    ff = {"kind": "moe", "expert": {"ff": s["ff"]},
+          "router": {"experts": s["experts"], "identity": 0, "top": s["top"], "groups": {"count": 4, "keep": 2}}}
+    layers = [dict(rec if i % 2 == 0 else att, mlp=ff) for i in range(s["layers"])]
+    return {"architecture": "Gazutar", "vocab": s["vocab"], "width": s["width"], "logit_scale": 1.0, "norm": {"eps": 1e-6},
+            "layers": layers}
+
+
+def qwen3_moe_config(s: dict) -> dict:
+    return dict(architectures=["Qwen3MoeForCausalLM"], model_type="qwen3_moe", hidden_size=s["width"],
+                num_hidden_layers=s["layers"], num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"],
+                head_dim=s["dim"], intermediate_size=4 * s["width"], vocab_size=s["vocab"], max_position_embeddings=8192,
+                rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False, attention_bias=False, hidden_act="silu",
+                torch_dtype="bfloat16", bos_token_id=0, eos_token_id=s["vocab"] - 1, num_experts=s["experts"],
+                num_experts_per_tok=s["top"], moe_intermediate_size=s["ff"], decoder_sparse_step=1, mlp_only_layers=[],
+                norm_topk_prob=True)
+
+
+def decode_weight_bytes(s: dict, batch: int, gazutar: bool) -> float:
+    """bf16 weight bytes one decode step of `batch` rows streams: projections, the experts the rows can reach, head."""
+    W, D, H, G = s["width"], s["dim"], s["heads"], s["kv_heads"]
+    experts_hit = min(s["experts"], batch * s["top"])
+    ff = experts_hit * 3 * W * s["ff"] + s["experts"] * W
+    if gazutar:
+        att = W * (2 * H * D + 2 * G * D) + H * D * W                 # q, g, k, v, o
+        r = W // 16
+        rec = W * (2 * G * D + H * D) + W * (2 * r + H) + r * 2 * H * D + H * D * W
+        mix = (s["layers"] // 2) * (att + rec)
+    else:
+        mix = s["layers"] * (W * (H * D + 2 * G * D) + H * D * W)
+    return 2.0 * (mix + s["layers"] * ff + s["vocab"] * W)
+
+
+def run_model(cfg: dict, batch: int, prompt_len: int, steps: int, warmup: int, **engine_kw) -> dict:
+    import torch
+
+    from nanovllm import LLM, SamplingParams
+
+    block = 64
+    blocks = batch * ((prompt_len + steps + warmup + 8) // block + 2) + 8
+    llm = LLM.from_config_dict(cfg, kvcache_block_size=block, max_num_seqs=batch, max_model_len=2 * prompt_len + 256,
+                               max_num_batched_tokens=8192, num_kvcache_blocks=blocks, synthetic_seed=0, sampling_seed=0,
+                               warmup=False, **engine_kw)
+    try:
+        vocab = llm._vocab()
+        rng = random.Random(0)
+        def prefill_all(max_tokens: int):
+            sp = SamplingParams(temperature=1.0, max_tokens=max_tokens, ignore_eos=True, greedy=True)
+            seqs = [llm.add_request([rng.randrange(vocab) for _ in range(prompt_len)], sp) for _ in range(batch)]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            while any(s.num_completion_tokens == 0 for s in seqs):
+                llm.step()
+            torch.cuda.synchronize()
+            return seqs, time.perf_counter() - t0
+
+        for _ in range(2):                           # two untimed passes: allocator growth, steps captured on second sight
+            prefill_all(2)
+            while not llm.is_finished():
+                llm.step()
+        seqs, t_prefill = prefill_all(steps + warmup + 4)
+        for _ in range(warmup):
+            llm.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            llm.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        runner = llm.model_runner
+        served = ("eager launches (row steps)" if getattr(runner, "hybrid", False) and not getattr(runner, "row_graphs", None)
+                  else "captured steps (hipGraph)")
+        return {"prefill_tok_s": batch * prompt_len / t_prefill, "prefill_ms": t_prefill * 1e3,
+                "decode_tok_s": batch * steps / dt, "ms_per_decode_step": dt / steps * 1e3, "served_as": served}
+    finally:
+        llm.exit()
+
+
+def main(args) -> dict:
+    batch, prompt_len = 32, 1024
+    out = {"metric": "design_throughput", "design": "gazutar", "closest_model": "Qwen3MoeForCausalLM", "unit": "tokens/s",
+           "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
+    for name, s in SIZES.items():
+        entry = {"shape": s}
+        for label, cfg, is_g in (("gazutar", gazutar_config(s), True), ("qwen3_moe", qwen3_moe_config(s), False)):
+            r = run_model(cfg, batch, prompt_len, args.steps, args.warmup)
+            wb = decode_weight_bytes(s, batch, is_g)
+            r["decode_weight_bytes"] = wb
+            r["decode_weight_roofline_frac"] = wb / (r["ms_per_decode_step"] * 1e-3) / HBM_BYTES_PER_S
+            entry[label] = r
+        entry["gazutar_vs_qwen3_moe"] = {k: entry["gazutar"][k] / entry["qwen3_moe"][k] for k in ("prefill_tok_s", "decode_tok_s")}
+        out["sizes"][name] = entry
+    print(json.dumps(out), flush=True)
+    return out

@@ -25,6 +25,8 @@
 // dtypes: the bf16 mode differs only in the dtype of the WEIGHTS and of the K/V cache.
 // A step's rows are described by cu_q [n_seqs + 1] (row range of each sequence) and kv_lens [n_seqs] (the sequence's
 // length INCLUDING this step's rows): row r of sequence s sits at position kv_lens[s] - (cu_q[s+1] - cu_q[s]) + r.
+#include <atomic>
+
 #include "mi_common.hpp"
 
 namespace mi {
@@ -525,10 +527,12 @@ extern "C" int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_o
   const int threads = ((D > Dv ? D : Dv) + 63) / 64 * 64;
   const size_t lds = ((size_t)D * Dv + 3 * (size_t)D + 16) * sizeof(float);
   if (threads > 512 || lds > 160 * 1024 - 512) return MI_EUNSUPPORTED;
-  if (lds > 48 * 1024) {
+  static std::atomic<size_t> lds_allowed{48 * 1024};  // raised once per size, outside any stream capture's path
+  if (lds > lds_allowed.load(std::memory_order_relaxed)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(channel_delta_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return MI_ERUNTIME;
+    lds_allowed.store(lds, std::memory_order_relaxed);
   }
   hipLaunchKernelGGL(channel_delta_kernel, dim3(n_seqs, H), dim3(threads), lds, S(stream), qkv, ld, q_off, k_off, v_off,
                      beta_pre, ld_beta, decay_pre, ld_decay, dt_bias, a_log, gate_pre, ld_gate, norm_w, state, cu_q,

@@ -198,6 +198,17 @@ class ModelRunner(RowSteps):
             self.graph_samples, self.graph_logits, self.prefill_graph_logits = set(), {}, {}
             self.tokens_dev = torch.zeros(config.max_num_seqs, dtype=torch.int64, device=self.device)
             self.prefill_graph_replays = 0
+            self.row_graphs, self.row_graph_logits = {}, {}
+            if config.use_graphs:
+                try:
+                    self.capture_row_graphs()
+                except Exception as e:
+                    import warnings
+
+                    warnings.warn(f"hipGraph capture of the decode steps failed ({e!r}); decoding eagerly")
+                    self.row_graphs.clear()
+                    self.row_graph_logits.clear()
+                    reset_context()
             return
         self.allocate_kv_cache()
         self._alloc_staging()
@@ -296,6 +307,9 @@ class ModelRunner(RowSteps):
         self.graph_logits.clear()
         self.prefill_graphs.clear()
         self.prefill_graph_logits.clear()
+        if self.hybrid:
+            self.row_graphs.clear()
+            self.row_graph_logits.clear()
         torch.cuda.synchronize()
         if self.channel is not None:
             if not abort:

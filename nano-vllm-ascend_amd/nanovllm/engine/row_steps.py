@@ -32,7 +32,8 @@ class RowSteps:
             cfg.num_kvcache_blocks = int(budget) // per_block
         assert cfg.num_kvcache_blocks > 1, "no memory left for the K/V pages"
         self.n_state_slots = n_slots
-        self.model.bind_cache(cfg.num_kvcache_blocks, self.block_size, n_slots, self.dtype, self.device)
+        # (one slot more than the scheduler hands out: the padded rows of a captured step write their state there)
+        self.model.bind_cache(cfg.num_kvcache_blocks, self.block_size, n_slots + 1, self.dtype, self.device)
 
     def _alloc_row_staging(self):
         nbytes = 1 << 16
@@ -118,14 +119,114 @@ class RowSteps:
         reset_context()
         return logits
 
+    # ------------------------------------------------------------------ captured decode steps
+    def _row_graph_layout(self):
+        cfg = self.config
+        B = cfg.max_num_seqs
+        cols = -(-cfg.max_model_len // self.block_size)
+        off, spans = 0, {}
+        for name, nbytes in (("ids", 8 * B), ("want", 8 * B), ("slots", 4 * B), ("cu", 4 * (B + 1)), ("kv", 4 * B),
+                             ("state", 4 * B), ("tables", 4 * B * cols)):
+            spans[name] = (off, nbytes)
+            off += (nbytes + 15) // 16 * 16
+
+        def views(buf):
+            def v(name, dtype, shape):
+                o, n = spans[name]
+                return buf[o:o + n].view(dtype).view(shape)
+            return {"ids": v("ids", torch.int64, (B,)), "want": v("want", torch.int64, (B,)),
+                    "slots": v("slots", torch.int32, (B,)), "cu": v("cu", torch.int32, (B + 1,)),
+                    "kv": v("kv", torch.int32, (B,)), "state": v("state", torch.int32, (B,)),
+                    "tables": v("tables", torch.int32, (B, cols))}
+        return off, cols, views
+
+    @torch.inference_mode()
+    def capture_row_graphs(self):
+        """Decode steps - one row per sequence - of the batch buckets 1, 2, 4, ..., max_num_seqs as hipGraphs (the
+        counterpart of ModelRunner.capture_decode_graphs for the row-step path).  The step's metadata sits at fixed
+        addresses of one static device buffer; padded rows are token 0 of a one-token sequence that stores no K/V row
+        (slot -1), reads the reserved last page and keeps its state in the spare slot.  The graph ends in the fp32
+        logits of every row; sampling stays outside."""
+        from nanovllm.engine.model_runner import CAPTURE_MODE, graph_buckets
+
+        cfg = self.config
+        nbytes, cols, views = self._row_graph_layout()
+        self._rg_cols = cols
+        self._rg_dev_buf = torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
+        self._rg_dev = views(self._rg_dev_buf)
+        self._rg_host_bufs = [torch.zeros(nbytes, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
+        self._rg_hosts = [{k: t.numpy() for k, t in views(b).items()} for b in self._rg_host_bufs]
+        self._rg_events = [None, None]
+        self._rg_flip = 0
+        d, pool = self._rg_dev, None
+        for bs in reversed(graph_buckets(cfg.max_num_seqs)):
+            self._stage_row_graph([], bs)
+            set_context(True, cu_seqlens_q=d["cu"][:bs + 1], kv_lens=d["kv"][:bs], slot_mapping=d["slots"][:bs],
+                        block_tables=d["tables"][:bs], block_size=self.block_size, state_slots=d["state"][:bs],
+                        max_seqlen_q=1, max_seqlen_k=cfg.max_model_len)
+
+            def body(bs=bs):
+                return self.model.compute_logits(self.model(d["ids"][:bs]))
+
+            side = torch.cuda.Stream(device=self.device)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):  # warm-up run outside capture
+                body()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=pool, capture_error_mode=CAPTURE_MODE):
+                logits = body()
+            pool = pool or graph.pool()
+            self.row_graphs[bs] = graph
+            self.row_graph_logits[bs] = logits
+        reset_context()
+        torch.cuda.synchronize()
+
+    def _stage_row_graph(self, seqs, bucket: int) -> None:
+        """Metadata of a decode step (every sequence's last token) at the static buffer's addresses, padded to the bucket."""
+        self._rg_flip ^= 1
+        b = self._rg_flip
+        if self._rg_events[b] is not None:
+            self._rg_events[b].synchronize()
+        h, bs, real = self._rg_hosts[b], self.block_size, len(seqs)
+        h["cu"][:] = np.arange(h["cu"].shape[0], dtype=np.int32)
+        h["want"][:] = np.arange(h["want"].shape[0], dtype=np.int64)
+        for i, s in enumerate(seqs):
+            n = len(s)
+            assert s.state_slot >= 0 and len(s.block_table) * bs >= n and len(s.block_table) <= self._rg_cols
+            h["ids"][i] = s.last_token
+            h["slots"][i] = s.block_table[(n - 1) // bs] * bs + (n - 1) % bs
+            h["kv"][i] = n
+            h["state"][i] = s.state_slot
+            h["tables"][i, :len(s.block_table)] = s.block_table
+        h["ids"][real:bucket] = 0
+        h["slots"][real:bucket] = -1
+        h["kv"][real:bucket] = 1
+        h["state"][real:bucket] = self.n_state_slots          # the spare slot
+        h["tables"][real:bucket, 0] = self.config.num_kvcache_blocks - 1   # the reserved page
+        self._rg_dev_buf.copy_(self._rg_host_bufs[b], non_blocking=True)
+        ev = self._rg_events[b] or torch.cuda.Event()
+        ev.record()
+        self._rg_events[b] = ev
+
     def run_hybrid(self, seqs, is_prefill: bool) -> list[int]:
         """ModelRunner.run for a hybrid model: the scheduler's prefill step (whole prompts; a preempted sequence comes back
         with its completion tokens and is recomputed from position 0, its state from zero) or decode step as row runs,
         then the framework's sampler on the last rows."""
-        runs = [(s, 0, len(s)) if is_prefill else (s, len(s) - 1, 1) for s in seqs]
-        logits = self.run_rows(runs)
-        self.last_logits = logits
         real = len(seqs)
+        bucket = None if is_prefill else next((b for b in sorted(self.row_graphs) if b >= real), None)
+        if bucket is not None:
+            self._stage_row_graph(seqs, bucket)
+            self.row_graphs[bucket].replay()
+            logits = self.row_graph_logits[bucket][:real]
+            for s in seqs:
+                s.num_computed_tokens = len(s)
+            self._steps_run += 1
+        else:
+            runs = [(s, 0, len(s)) if is_prefill else (s, len(s) - 1, 1) for s in seqs]
+            logits = self.run_rows(runs)
+        self.last_logits = logits
         temps = torch.tensor([0.0 if s.greedy else s.temperature for s in seqs], dtype=torch.float32).to(self.device)
         # the sampler reads bf16 logits in rows of a multiple of 8 elements (layers/sampler.py)
         vocab = logits.shape[1]

@@ -301,6 +301,30 @@ def test_greedy_generation_through_llm(mixed_model, dtype):
         llm.exit()
 
 
+def test_captured_decode_steps_equal_eager(mixed_model):
+    """The engine's decode steps replay hipGraphs padded to a batch bucket (here 3 live requests in the bucket of 4, the
+    padded row writing the spare state slot): same tokens and, for the real rows, the same logits as eager launches -
+    over several replays with the engine's own eager prefill steps between them."""
+    from nanovllm import LLM, SamplingParams
+
+    cfg, w, d = mixed_model
+    prompts = [tokens_of(n, cfg["vocab"], 70 + n) for n in (9, 31, 16, 5, 22)]
+    sp = SamplingParams(max_tokens=10, greedy=True, ignore_eos=True)
+    runs, logits = [], []
+    for eager in (True, False):
+        llm = LLM(d, dtype="float32", kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=4, max_model_len=128,
+                  max_num_batched_tokens=128, warmup=False, enforce_eager=eager)
+        try:
+            assert bool(llm.model_runner.row_graphs) == (not eager)
+            runs.append([o["token_ids"] for o in llm.generate(prompts[:3], sp, use_tqdm=False)])
+            runs[-1] += [o["token_ids"] for o in llm.generate(prompts[3:], sp, use_tqdm=False)]
+            logits.append(llm.model_runner.last_logits.float().cpu().clone())
+        finally:
+            llm.exit()
+    assert runs[0] == runs[1]
+    assert rel_err(logits[1], logits[0]) <= CUT_BAR
+
+
 def test_preempted_request_is_recomputed(mixed_model):
     """So few pages that a running request is preempted: it gives its pages and slot back, comes back with its completion
     tokens and is recomputed from position 0 - the tokens are the ones it gets with room for everybody."""
