@@ -688,7 +688,10 @@ int mi_causal_conv_silu(const float* x, int64_t ldx, const float* w, int taps, c
                         int64_t ldy, mi_stream stream);
 int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, const int32_t* cu_q,
                          const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int channels, mi_stream stream);
-/* Gated delta rule with a decay per (head, key channel); state [slots][H][D][Dv] fp32.  Per row and head h (q / k
+/* Floats of recurrent state one sequence slot holds for mi_channel_delta (the kernel's own thread-order layout), or
+ * -1 when D is beyond the compiled kernels (D <= 256).  Host only. */
+int64_t mi_channel_delta_state_elems(int H, int D, int Dv);
+/* Gated delta rule with a decay per (head, key channel); state [slots][mi_channel_delta_state_elems] fp32.  Per row and head h (q / k
  * head h / (H / G)): q, k <- unit vectors (x / sqrt(sum x^2 + 1e-6)), q / sqrt(D); g = exp(-exp(a_log[h]) *
  * softplus(decay_pre[row][h*D..] + dt_bias[h*D..])); beta = sigmoid(beta_pre[row][h]);
  * S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q;
@@ -696,8 +699,8 @@ int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, co
 int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_off, const float* beta_pre,
                      int64_t ld_beta, const float* decay_pre, int64_t ld_decay, const float* dt_bias,
                      const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w, float* state,
-                     const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int H, int G,
-                     int D, int Dv, float eps, float* out, int64_t ldo, mi_stream stream);
+                     const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int n_rows, int H,
+                     int G, int D, int Dv, float eps, float* out, int64_t ldo, mi_stream stream);
 /* Router with expert groups: scores = softmax(logits) over n_outputs; choice = scores + correction; only the
  * `keep` of `n_groups` equal groups of neighbours with the largest best choice are eligible; ids = the top_k
  * eligible outputs by choice (descending), weights = their scores (not renormalised).  n_outputs <= 512. */

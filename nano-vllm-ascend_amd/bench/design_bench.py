@@ -109,15 +109,22 @@ def main(args) -> dict:
     out = {"metric": "design_throughput", "design": "gazutar", "closest_model": "Qwen3MoeForCausalLM", "unit": "tokens/s",
            "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
            "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
+    only_sizes = [x for x in getattr(args, "design_sizes", "").split(",") if x]
+    only_models = [x for x in getattr(args, "design_models", "").split(",") if x]
     for name, s in SIZES.items():
+        if only_sizes and name not in only_sizes:
+            continue
         entry = {"shape": s}
         for label, cfg, is_g in (("gazutar", gazutar_config(s), True), ("qwen3_moe", qwen3_moe_config(s), False)):
+            if only_models and label not in only_models:
+                continue
             r = run_model(cfg, batch, prompt_len, args.steps, args.warmup)
             wb = decode_weight_bytes(s, batch, is_g)
             r["decode_weight_bytes"] = wb
             r["decode_weight_roofline_frac"] = wb / (r["ms_per_decode_step"] * 1e-3) / HBM_BYTES_PER_S
             entry[label] = r
-        entry["gazutar_vs_qwen3_moe"] = {k: entry["gazutar"][k] / entry["qwen3_moe"][k] for k in ("prefill_tok_s", "decode_tok_s")}
+        if "gazutar" in entry and "qwen3_moe" in entry:
+            entry["gazutar_vs_qwen3_moe"] = {k: entry["gazutar"][k] / entry["qwen3_moe"][k] for k in ("prefill_tok_s", "decode_tok_s")}
         out["sizes"][name] = entry
     print(json.dumps(out), flush=True)
     return out

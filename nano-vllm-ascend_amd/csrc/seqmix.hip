@@ -16,7 +16,7 @@
 //   mi_channel_delta            gated delta rule with one decay per head AND key channel:
 //                               S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 //                               with unit-norm q / k, per-head RMS norm of o, sigmoid gate; the fp32 state lives in a
-//                               per-sequence slot and is carried from step to step
+//                               per-sequence slot (mi_channel_delta_state_elems floats) and is carried from step to step
 //   mi_route_grouped            router of a sparse feed-forward: softmax scores, additive choice correction, choice
 //                               restricted to the best groups of experts, top-k; weights = un-renormalised scores
 //   mi_moe_combine_f32          out[t] = sum_k w[t][k] * (identity expert ? h[t] : y[t * top_k + k])
@@ -25,8 +25,6 @@
 // dtypes: the bf16 mode differs only in the dtype of the WEIGHTS and of the K/V cache.
 // A step's rows are described by cu_q [n_seqs + 1] (row range of each sequence) and kv_lens [n_seqs] (the sequence's
 // length INCLUDING this step's rows): row r of sequence s sits at position kv_lens[s] - (cu_q[s+1] - cu_q[s]) + r.
-#include <atomic>
-
 #include "mi_common.hpp"
 
 namespace mi {
@@ -267,85 +265,130 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(const float* __r
 // ---------------------------------------------------------------------------------------------------------------
 // gated delta rule, decay per head and key channel
 // ---------------------------------------------------------------------------------------------------------------
-// One workgroup per (sequence, head), walking the sequence's rows of this step in order.  The state S [D][Dv] stays in
-// LDS for the whole walk (thread j owns column j: S^T k, the rank-one update and S^T q are per-column loops without any
-// exchange), read from / written to the sequence's slot.  Threads i < D prepare the row's key-channel vectors (unit q
-// and k, decay), threads j < Dv the value side.  blockDim = max(D, Dv) rounded up to 64.
-__global__ void channel_delta_kernel(const float* __restrict__ qkv, int64_t ld, int q_off, int k_off, int v_off,
-                                     const float* __restrict__ beta_pre, int64_t ld_beta,
-                                     const float* __restrict__ decay_pre, int64_t ld_decay,
-                                     const float* __restrict__ dt_bias, const float* __restrict__ a_log,
-                                     const float* __restrict__ gate_pre, int64_t ld_gate,
-                                     const float* __restrict__ norm_w, float* __restrict__ state,
-                                     const int32_t* __restrict__ cu_q, const int32_t* __restrict__ kv_lens,
-                                     const int32_t* __restrict__ slot_ids, int H, int G, int D, int Dv, float eps,
-                                     float* __restrict__ out, int64_t ldo) {
-  extern __shared__ float smem[];
-  float* S = smem;                 // [D][Dv]
-  float* qv = S + D * Dv;          // [D]
-  float* kv = qv + D;              // [D]
-  float* gv = kv + D;              // [D]
-  float* red = gv + D;             // [16]
-  const int s = blockIdx.x, h = blockIdx.y;
-  const int tid = threadIdx.x, nthr = blockDim.x, nwaves = nthr >> 6;
+// The columns of S (one per value channel) never exchange anything: S^T k, the rank-one update and S^T q are per-column
+// sums over the key channels.  One workgroup = 64 value columns of one (sequence, head); a column is held by FOUR lanes
+// (quad), each keeping DR of the (padded) 4 * DR key channels of it in registers for the whole walk over the sequence's
+// rows of this step - lane r of the quad owns the channels (4 jj + r) * 4 + e, so that a quad's LDS reads of the row's
+// k / q / decay vectors are four consecutive 16-byte pieces and the two sums over the key channels end in two DPP steps
+// inside the quad.  Rows are prepared 16 at a time by all 256 threads (unit q and k, decay, sigmoid of beta, the value
+// columns) into LDS; between two preparations the walk needs no barrier.  The state is kept in memory in THREAD order
+// ([slot][head][column block][DR][256]: register ii of thread t at ii * 256 + t), read and written fully coalesced and
+// touched by nothing else.  The read-out is written raw; delta_finish_kernel applies the per-head RMS norm and gate.
+constexpr int kDeltaCols = 64, kDeltaRows = 16;
+
+template <int DR>
+__global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restrict__ qkv, int64_t ld, int q_off,
+                                                            int k_off, int v_off, const float* __restrict__ beta_pre,
+                                                            int64_t ld_beta, const float* __restrict__ decay_pre,
+                                                            int64_t ld_decay, const float* __restrict__ dt_bias,
+                                                            const float* __restrict__ a_log, float* __restrict__ state,
+                                                            const int32_t* __restrict__ cu_q,
+                                                            const int32_t* __restrict__ kv_lens,
+                                                            const int32_t* __restrict__ slot_ids, int H, int G, int D,
+                                                            int Dv, float* __restrict__ out, int64_t ldo) {
+  constexpr int DP = 4 * DR;  // padded key channels
+  __shared__ __attribute__((aligned(16))) float qs[kDeltaRows][DP];
+  __shared__ __attribute__((aligned(16))) float ks[kDeltaRows][DP];
+  __shared__ __attribute__((aligned(16))) float gs[kDeltaRows][DP];
+  __shared__ float vs[kDeltaRows][kDeltaCols];
+  __shared__ float bs[kDeltaRows];
+  const int s = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
+  const int tid = threadIdx.x, r = tid & 3, col = tid >> 2;
+  const int c = cb * kDeltaCols + col;
   const int r0 = cu_q[s], n = cu_q[s + 1] - r0;
   if (n == 0) return;
   const int start = kv_lens[s] - n;
   const int kvh = h / (H / G);
-  float* slot = state + ((int64_t)slot_ids[s] * H + h) * D * Dv;
-  for (int e = tid; e < D * Dv; e += nthr) S[e] = start > 0 ? slot[e] : 0.f;
+  float* slot = state + (((int64_t)slot_ids[s] * H + h) * gridDim.z + cb) * DR * 256;
+  float st[DR];
+#pragma unroll
+  for (int ii = 0; ii < DR; ++ii) st[ii] = start > 0 ? slot[ii * 256 + tid] : 0.f;
   const float decay_rate = expf(a_log[h]);
   const float q_scale = 1.f / sqrtf((float)D);
-  __syncthreads();
-  for (int r = 0; r < n; ++r) {
-    const int64_t row = r0 + r;
-    // key side: sums of squares of q and k over D (fixed order: wave butterfly, then the waves in order)
-    float qr = 0.f, kr = 0.f;
-    if (tid < D) {
-      qr = qkv[row * ld + q_off + kvh * D + tid];
-      kr = qkv[row * ld + k_off + kvh * D + tid];
+  const int pt = tid >> 4, ps = tid & 15;  // preparation: 16 lanes per row
+  for (int c0 = 0; c0 < n; c0 += kDeltaRows) {
+    __syncthreads();  // the previous rows' vectors have been consumed
+    {
+      const bool live = c0 + pt < n;
+      const int64_t row = r0 + c0 + (live ? pt : 0);
+      float sq = 0.f, sk = 0.f;
+      for (int i = ps; i < D; i += 16) {
+        const float qv = qkv[row * ld + q_off + kvh * D + i], kv = qkv[row * ld + k_off + kvh * D + i];
+        sq = fmaf(qv, qv, sq);
+        sk = fmaf(kv, kv, sk);
+      }
+      sq = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>(sq))));
+      sk = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>(sk))));
+      const float nq = q_scale / sqrtf(sq + 1e-6f), nk = 1.f / sqrtf(sk + 1e-6f);
+      for (int i = ps; i < DP; i += 16) {
+        float qv = 0.f, kv = 0.f, gv = 0.f;
+        if (i < D && live) {
+          qv = qkv[row * ld + q_off + kvh * D + i] * nq;
+          kv = qkv[row * ld + k_off + kvh * D + i] * nk;
+          gv = expf(-decay_rate * softplus_f(decay_pre[row * ld_decay + h * D + i] + dt_bias[h * D + i]));
+        }
+        qs[pt][i] = qv, ks[pt][i] = kv, gs[pt][i] = gv;
+      }
+      for (int e = ps; e < kDeltaCols; e += 16) {
+        const int cc = cb * kDeltaCols + e;
+        vs[pt][e] = (live && cc < Dv) ? qkv[row * ld + v_off + h * Dv + cc] : 0.f;
+      }
+      if (ps == 0) bs[pt] = live ? sigmoid_f(beta_pre[row * ld_beta + h]) : 0.f;
     }
-    const float sq = wave_sum(qr * qr), sk = wave_sum(kr * kr);
-    if ((tid & 63) == 0) red[tid >> 6] = sq, red[8 + (tid >> 6)] = sk;
     __syncthreads();
-    float tq = 0.f, tk = 0.f;
-    for (int wv = 0; wv < nwaves; ++wv) tq += red[wv], tk += red[8 + wv];
-    if (tid < D) {
-      qv[tid] = qr / sqrtf(tq + 1e-6f) * q_scale;
-      kv[tid] = kr / sqrtf(tk + 1e-6f);
-      const float dt = softplus_f(decay_pre[row * ld_decay + h * D + tid] + dt_bias[h * D + tid]);
-      gv[tid] = expf(-decay_rate * dt);
-    }
-    __syncthreads();
-    float o = 0.f;
-    if (tid < Dv) {
+    const int nt = min(kDeltaRows, n - c0);
+    for (int t = 0; t < nt; ++t) {
+      const float4* g4 = reinterpret_cast<const float4*>(gs[t]);
+      const float4* k4 = reinterpret_cast<const float4*>(ks[t]);
+      const float4* q4 = reinterpret_cast<const float4*>(qs[t]);
       float dot = 0.f;
-      for (int i = 0; i < D; ++i) {
-        const float sv = S[i * Dv + tid] * gv[i];
-        S[i * Dv + tid] = sv;
-        dot = fmaf(sv, kv[i], dot);
+#pragma unroll
+      for (int jj = 0; jj < DR / 4; ++jj) {
+        const float4 gv = g4[jj * 4 + r], kv = k4[jj * 4 + r];
+        st[jj * 4 + 0] *= gv.x, st[jj * 4 + 1] *= gv.y, st[jj * 4 + 2] *= gv.z, st[jj * 4 + 3] *= gv.w;
+        dot = fmaf(st[jj * 4 + 0], kv.x, dot);
+        dot = fmaf(st[jj * 4 + 1], kv.y, dot);
+        dot = fmaf(st[jj * 4 + 2], kv.z, dot);
+        dot = fmaf(st[jj * 4 + 3], kv.w, dot);
       }
-      const float beta = sigmoid_f(beta_pre[row * ld_beta + h]);
-      const float u = beta * (qkv[row * ld + v_off + h * Dv + tid] - dot);
-      for (int i = 0; i < D; ++i) {
-        const float sv = fmaf(kv[i], u, S[i * Dv + tid]);
-        S[i * Dv + tid] = sv;
-        o = fmaf(sv, qv[i], o);
+      dot = xor_sum<2>(xor_sum<1>(dot));
+      const float u = bs[t] * (vs[t][col] - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int jj = 0; jj < DR / 4; ++jj) {
+        const float4 kv = k4[jj * 4 + r], qv = q4[jj * 4 + r];
+        st[jj * 4 + 0] = fmaf(kv.x, u, st[jj * 4 + 0]);
+        st[jj * 4 + 1] = fmaf(kv.y, u, st[jj * 4 + 1]);
+        st[jj * 4 + 2] = fmaf(kv.z, u, st[jj * 4 + 2]);
+        st[jj * 4 + 3] = fmaf(kv.w, u, st[jj * 4 + 3]);
+        o = fmaf(st[jj * 4 + 0], qv.x, o);
+        o = fmaf(st[jj * 4 + 1], qv.y, o);
+        o = fmaf(st[jj * 4 + 2], qv.z, o);
+        o = fmaf(st[jj * 4 + 3], qv.w, o);
       }
+      o = xor_sum<2>(xor_sum<1>(o));
+      if (r == 0 && c < Dv) out[(int64_t)(r0 + c0 + t) * ldo + h * Dv + c] = o;
     }
-    const float so = wave_sum(o * o);
-    __syncthreads();  // (red's previous contents have been read by everyone; qv / kv / gv are free again after this)
-    if ((tid & 63) == 0) red[tid >> 6] = so;
-    __syncthreads();
-    float to = 0.f;
-    for (int wv = 0; wv < nwaves; ++wv) to += red[wv];
-    if (tid < Dv) {
-      const float rstd = 1.f / sqrtf(to / (float)Dv + eps);
-      out[row * ldo + h * Dv + tid] = o * rstd * norm_w[tid] * sigmoid_f(gate_pre[row * ld_gate + h * Dv + tid]);
-    }
-    __syncthreads();
   }
-  for (int e = tid; e < D * Dv; e += nthr) slot[e] = S[e];
+#pragma unroll
+  for (int ii = 0; ii < DR; ++ii) slot[ii * 256 + tid] = st[ii];
+}
+
+// out[row][h] <- out / rms(out over Dv) * norm_w * sigmoid(gate): one wave per (row, head), in place
+__global__ __launch_bounds__(256) void delta_finish_kernel(float* __restrict__ out, int64_t ldo,
+                                                           const float* __restrict__ gate_pre, int64_t ld_gate,
+                                                           const float* __restrict__ norm_w, int n_rows, int H, int Dv,
+                                                           float eps) {
+  const int lane = threadIdx.x & 63;
+  const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (wid >= n_rows * H) return;
+  const int row = wid / H, h = wid % H;
+  float* o = out + (int64_t)row * ldo + h * Dv;
+  float sq = 0.f;
+  for (int d = lane; d < Dv; d += 64) sq = fmaf(o[d], o[d], sq);
+  const float rstd = 1.f / sqrtf(wave_sum(sq) / (float)Dv + eps);
+  for (int d = lane; d < Dv; d += 64)
+    o[d] = o[d] * rstd * norm_w[d] * sigmoid_f(gate_pre[(int64_t)row * ld_gate + h * Dv + d]);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -514,29 +557,38 @@ extern "C" int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float
   return check_launch();
 }
 
+static int delta_dr(int D) { return D <= 64 ? 16 : D <= 128 ? 32 : D <= 256 ? 64 : 0; }
+
+extern "C" int64_t mi_channel_delta_state_elems(int H, int D, int Dv) {
+  const int dr = delta_dr(D);
+  if (H < 1 || D < 1 || Dv < 1 || dr == 0) return -1;
+  return (int64_t)H * ((Dv + kDeltaCols - 1) / kDeltaCols) * dr * 256;
+}
+
 extern "C" int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_off, const float* beta_pre,
                                 int64_t ld_beta, const float* decay_pre, int64_t ld_decay, const float* dt_bias,
                                 const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w,
                                 float* state, const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids,
-                                int n_seqs, int H, int G, int D, int Dv, float eps, float* out, int64_t ldo,
+                                int n_seqs, int n_rows, int H, int G, int D, int Dv, float eps, float* out, int64_t ldo,
                                 mi_stream stream) {
   if (!qkv || !beta_pre || !decay_pre || !dt_bias || !a_log || !gate_pre || !norm_w || !state || !cu_q || !kv_lens ||
-      !slot_ids || !out || n_seqs < 1)
+      !slot_ids || !out || n_seqs < 1 || n_rows < 0)
     return MI_EINVAL;
   if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1) return MI_EINVAL;
-  const int threads = ((D > Dv ? D : Dv) + 63) / 64 * 64;
-  const size_t lds = ((size_t)D * Dv + 3 * (size_t)D + 16) * sizeof(float);
-  if (threads > 512 || lds > 160 * 1024 - 512) return MI_EUNSUPPORTED;
-  static std::atomic<size_t> lds_allowed{48 * 1024};  // raised once per size, outside any stream capture's path
-  if (lds > lds_allowed.load(std::memory_order_relaxed)) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(channel_delta_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return MI_ERUNTIME;
-    lds_allowed.store(lds, std::memory_order_relaxed);
-  }
-  hipLaunchKernelGGL(channel_delta_kernel, dim3(n_seqs, H), dim3(threads), lds, S(stream), qkv, ld, q_off, k_off, v_off,
-                     beta_pre, ld_beta, decay_pre, ld_decay, dt_bias, a_log, gate_pre, ld_gate, norm_w, state, cu_q,
-                     kv_lens, slot_ids, H, G, D, Dv, eps, out, ldo);
+  const int dr = delta_dr(D);
+  if (dr == 0 || n_seqs > 65535) return MI_EUNSUPPORTED;
+  if (n_rows == 0) return MI_OK;
+  const dim3 grid(n_seqs, H, (Dv + kDeltaCols - 1) / kDeltaCols), block(256);
+#define MI_DELTA(DR)                                                                                                  \
+  hipLaunchKernelGGL((channel_delta_kernel<DR>), grid, block, 0, S(stream), qkv, ld, q_off, k_off, v_off, beta_pre,     \
+                     ld_beta, decay_pre, ld_decay, dt_bias, a_log, state, cu_q, kv_lens, slot_ids, H, G, D, Dv, out, ldo)
+  if (dr == 16) MI_DELTA(16);
+  else if (dr == 32) MI_DELTA(32);
+  else MI_DELTA(64);
+#undef MI_DELTA
+  if (check_launch() != MI_OK) return MI_ELAUNCH;
+  hipLaunchKernelGGL(delta_finish_kernel, dim3((n_rows * H + 3) / 4), dim3(256), 0, S(stream), out, ldo, gate_pre,
+                     ld_gate, norm_w, n_rows, H, Dv, eps);
   return check_launch();
 }
 

@@ -121,7 +121,8 @@ class ChannelDeltaMixer(nn.Module):
         self.state = self.conv_state = torch.tensor([])
 
     def state_shapes(self, n_slots: int):
-        return (n_slots, self.H, self.D, self.Dv), (n_slots, max(self.taps - 1, 1), self.qkv.weight.shape[0])
+        return ((n_slots, ops.channel_delta_state_elems(self.H, self.D, self.Dv)),
+                (n_slots, max(self.taps - 1, 1), self.qkv.weight.shape[0]))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         ctx = get_context()

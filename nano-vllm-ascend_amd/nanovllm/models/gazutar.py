@@ -191,7 +191,7 @@ class GazutarForCausalLM(nn.Module):
         for l in self.layers:
             if l.kind == "channel_delta":
                 s, c = l.mix.state_shapes(1)
-                n += 4 * (s[1] * s[2] * s[3] + c[1] * c[2])
+                n += 4 * (s[1] + c[1] * c[2])
         return n
 
     def bind_cache(self, num_blocks: int, block_size: int, n_slots: int, dtype: torch.dtype, device) -> None:

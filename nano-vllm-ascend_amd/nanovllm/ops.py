@@ -1058,20 +1058,28 @@ def causal_conv_state(x, taps: int, state, cu_q, kv_lens, slot_ids) -> None:
                                    kv_lens.numel(), x.shape[1], stream()), "mi_causal_conv_state")
 
 
+def channel_delta_state_elems(H: int, D: int, Dv: int) -> int:
+    """Floats of recurrent state per sequence slot (the kernel keeps it in its own thread-order layout)."""
+    n = lib.mi_channel_delta_state_elems(H, D, Dv)
+    if n < 0:
+        raise _C.MiError(f"channel_delta: {D} key channels per head are beyond the compiled kernels (<= 256)")
+    return n
+
+
 def channel_delta(qkv, q_off: int, k_off: int, v_off: int, beta_pre, decay_pre, dt_bias, a_log, gate_pre, norm_w, state,
                   cu_q, kv_lens, slot_ids, H: int, G: int, D: int, Dv: int, eps: float) -> torch.Tensor:
     require_gpu(qkv, state)
     _f32(qkv, beta_pre, decay_pre, dt_bias, a_log, gate_pre, norm_w, state)
     _i32(cu_q, kv_lens, slot_ids)
     rows = qkv.shape[0]
-    assert state.is_contiguous() and state.shape[1:] == (H, D, Dv), state.shape
+    assert state.is_contiguous() and state.shape[1] == channel_delta_state_elems(H, D, Dv), state.shape
     assert beta_pre.shape == (rows, H) and decay_pre.shape == (rows, H * D) and gate_pre.shape == (rows, H * Dv)
     assert dt_bias.numel() == H * D and a_log.numel() == H and norm_w.numel() == Dv
     out = torch.empty((rows, H * Dv), dtype=_F32, device=qkv.device)
     check(lib.mi_channel_delta(ptr(qkv), qkv.stride(0), q_off, k_off, v_off, ptr(beta_pre), beta_pre.stride(0),
                                ptr(decay_pre), decay_pre.stride(0), ptr(dt_bias), ptr(a_log), ptr(gate_pre),
                                gate_pre.stride(0), ptr(norm_w), ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
-                               kv_lens.numel(), H, G, D, Dv, float(eps), ptr(out), out.stride(0), stream()),
+                               kv_lens.numel(), rows, H, G, D, Dv, float(eps), ptr(out), out.stride(0), stream()),
           "mi_channel_delta")
     return out
 
