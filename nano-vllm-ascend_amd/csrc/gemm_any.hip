@@ -44,6 +44,31 @@ __device__ __forceinline__ float w_load<uint16_t>(const uint16_t* p) { return bf
 __device__ __forceinline__ bool dev_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
 
+// eight consecutive operands as floats: one 16-byte (bf16) / two 16-byte (fp32) loads, or element-wise at an edge
+template <typename TW>
+__device__ __forceinline__ void load8(const TW* p, int n_valid, bool vec, float (&v)[8]);
+template <>
+__device__ __forceinline__ void load8<uint16_t>(const uint16_t* p, int n_valid, bool vec, float (&v)[8]) {
+  if (vec && n_valid >= 8) {
+    const u32x4 w = *reinterpret_cast<const u32x4*>(p);
+    v[0] = lo_bf(w[0]), v[1] = hi_bf(w[0]), v[2] = lo_bf(w[1]), v[3] = hi_bf(w[1]);
+    v[4] = lo_bf(w[2]), v[5] = hi_bf(w[2]), v[6] = lo_bf(w[3]), v[7] = hi_bf(w[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = i < n_valid ? bf2f(p[i]) : 0.f;
+  }
+}
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, int n_valid, bool vec, float (&v)[8]) {
+  if (vec && n_valid >= 8) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = i < n_valid ? p[i] : 0.f;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // exact kernel: 64 x 64 tile, 256 threads, 4 x 4 outputs per thread, k ascending
 // ---------------------------------------------------------------------------------------------------------------
@@ -116,12 +141,12 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
 
 // ---------------------------------------------------------------------------------------------------------------
 // MFMA kernel (bf16 weights): 64 x 64 tile, 4 waves as 2 x 2, each wave 32 x 32 = 2 x 2 fragments of 16 x 16,
-// K in steps of 32.  LDS holds the tile's x rows and weight rows as bf16 [64][32 + 8] (row stride 80 bytes: the eight
-// rows a quarter-wave reads start in different banks).
+// K in steps of 64 (a weight row's piece = one 128-byte line).  LDS holds the tile's x rows and weight rows as bf16
+// [64][64 + 8].
 // ---------------------------------------------------------------------------------------------------------------
 template <bool DUAL>
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
-  constexpr int BM = 64, BN = 64, BK = 32, LD = BK + 8;
+  constexpr int BM = 64, BN = 64, BK = 64, LD = BK + 8;
   __shared__ __attribute__((aligned(16))) uint16_t As[BM][LD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[DUAL ? 2 : 1][BN][LD];
   const int tid = threadIdx.x;
@@ -137,7 +162,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
   const int m0 = m_lo + blockIdx.y * BM;
   if (m0 >= m_hi) return;
   const int n0 = blockIdx.x * BN;
-  const int lr = tid >> 2, lk = (tid & 3) * 8;
+  const int lr = tid >> 2, lk = (tid & 3) * 16;  // this thread stages 16 consecutive k of one row: a row's 64 k = one 128-byte line of weights
   int64_t xrow = -1;
   if (m0 + lr < m_hi) xrow = a.x_rows ? a.x_rows[m0 + lr] : m0 + lr;
   const int wrow = n0 + lr < a.N ? n0 + lr : -1;
@@ -154,53 +179,56 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[d][i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < a.K; k0 += BK) {
-    const int k = k0 + lk;
-    // x: 8 floats -> 8 bf16 (round to nearest even)
-    float xv[8];
-    if (xrow >= 0 && x_vec && k + 8 <= a.K) {
-      const float4 p0 = *reinterpret_cast<const float4*>(a.x + xrow * a.ldx + k);
-      const float4 p1 = *reinterpret_cast<const float4*>(a.x + xrow * a.ldx + k + 4);
-      xv[0] = p0.x, xv[1] = p0.y, xv[2] = p0.z, xv[3] = p0.w, xv[4] = p1.x, xv[5] = p1.y, xv[6] = p1.z, xv[7] = p1.w;
-    } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) xv[i] = (xrow >= 0 && k + i < a.K) ? a.x[xrow * a.ldx + k + i] : 0.f;
-    }
-    u32x4 xp = {pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
-    *reinterpret_cast<u32x4*>(&As[lr][lk]) = xp;
+    for (int half = 0; half < 2; ++half) {
+      const int k = k0 + lk + half * 8;
+      float xv[8];
+      if (xrow >= 0) load8<float>(a.x + xrow * a.ldx + k, a.K - k, x_vec, xv);
+      else {
 #pragma unroll
-    for (int d = 0; d < (DUAL ? 2 : 1); ++d) {
-      const uint16_t* wp = (d ? w2 : w) + (int64_t)wrow * a.K + k;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (wrow >= 0) {
-        if (w_vec && k + 8 <= a.K) {
-          v = *reinterpret_cast<const u32x4*>(wp);
-        } else {
-          uint16_t e[8];
-#pragma unroll
-          for (int i = 0; i < 8; ++i) e[i] = k + i < a.K ? wp[i] : (uint16_t)0;
-          v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
-                    (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
-        }
+        for (int i = 0; i < 8; ++i) xv[i] = 0.f;
       }
-      *reinterpret_cast<u32x4*>(&Bs[d][lr][lk]) = v;
+      const u32x4 xp = {pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
+      *reinterpret_cast<u32x4*>(&As[lr][lk + half * 8]) = xp;
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d) {
+        const uint16_t* wp = (d ? w2 : w) + (int64_t)wrow * a.K + k;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (wrow >= 0 && k < a.K) {
+          if (w_vec && k + 8 <= a.K) {
+            v = *reinterpret_cast<const u32x4*>(wp);
+          } else {
+            uint16_t e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = k + i < a.K ? wp[i] : (uint16_t)0;
+            v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                      (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+          }
+        }
+        *reinterpret_cast<u32x4*>(&Bs[d][lr][lk + half * 8]) = v;
+      }
     }
     __syncthreads();
-    bf16x8 af[2], bfr[DUAL ? 2 : 1][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) af[i] = as_frag(*reinterpret_cast<const u32x4*>(&As[wm + i * 16 + fr][fk]));
-#pragma unroll
-    for (int d = 0; d < (DUAL ? 2 : 1); ++d)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) bfr[d][j] = as_frag(*reinterpret_cast<const u32x4*>(&Bs[d][wn + j * 16 + fr][fk]));
     // D[n][m] = sum_k W[n][k] X[m][k]: weights on the MFMA's row axis, so a lane's four results are four consecutive
     // FEATURES of one x row
 #pragma unroll
-    for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 af[2], bfr[DUAL ? 2 : 1][2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i) af[i] = as_frag(*reinterpret_cast<const u32x4*>(&As[wm + i * 16 + fr][ks * 32 + fk]));
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[d][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[d][j], af[i], acc[d][i][j], 0, 0, 0);
+          bfr[d][j] = as_frag(*reinterpret_cast<const u32x4*>(&Bs[d][wn + j * 16 + fr][ks * 32 + fk]));
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            acc[d][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[d][j], af[i], acc[d][i][j], 0, 0, 0);
+    }
     __syncthreads();
   }
   // fragment (i, j): x row = wm + i*16 + (lane & 15), features wn + j*16 + (lane >> 4) * 4 + r
@@ -216,14 +244,15 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
         const int n = n0 + wn + j * 16 + (lane >> 4) * 4 + r;
         if (n >= a.N) continue;
         float v = acc[0][i][j][r];
-        if (DUAL) v = silu_f(v) * acc[1][i][j][r];
+        if (DUAL) v = silu_f(v) * acc[DUAL ? 1 : 0][i][j][r];
         a.y[yrow * a.ldy + n] = v * a.alpha;
       }
   }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// few rows (decode): one wave per output feature; lanes take K in pieces of 8, ascending, then a butterfly
+// few rows: one wave per output feature and batch of MT rows (blockIdx.y); the lanes take K in pieces of 8, ascending,
+// 16-byte loads where the operands allow it, then a butterfly over the lanes
 // ---------------------------------------------------------------------------------------------------------------
 template <typename TW, int MT, bool DUAL>
 __global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
@@ -238,38 +267,36 @@ __global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
     w += (int64_t)blockIdx.z * a.N * a.K;
     if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
   }
-  if (n >= a.N) return;  // (whole waves: the reductions below see all 64 lanes)
-  for (int m0 = m_lo; m0 < m_hi; m0 += MT) {
-    float acc[DUAL ? 2 : 1][MT] = {};
-    int64_t xr[MT];
+  const int m0 = m_lo + blockIdx.y * MT;
+  if (n >= a.N || m0 >= m_hi) return;  // (whole waves: the reductions below see all 64 lanes)
+  const bool w_vec = a.K % 8 == 0 && dev_aligned16(a.w) && (!DUAL || dev_aligned16(a.w2));
+  const bool x_vec = a.ldx % 4 == 0 && dev_aligned16(a.x);
+  float acc[DUAL ? 2 : 1][MT] = {};
+  int64_t xr[MT];
 #pragma unroll
-    for (int r = 0; r < MT; ++r) xr[r] = m0 + r < m_hi ? (a.x_rows ? a.x_rows[m0 + r] : m0 + r) : -1;
-    for (int k0 = lane * 8; k0 < a.K; k0 += 64 * 8) {
-      float wv[DUAL ? 2 : 1][8];
-#pragma unroll
-      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          wv[d][i] = k0 + i < a.K ? w_load<TW>((d ? w2 : w) + (int64_t)n * a.K + k0 + i) : 0.f;
-#pragma unroll
-      for (int r = 0; r < MT; ++r) {
-        if (xr[r] < 0) continue;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float xv = k0 + i < a.K ? a.x[xr[r] * a.ldx + k0 + i] : 0.f;
-#pragma unroll
-          for (int d = 0; d < (DUAL ? 2 : 1); ++d) acc[d][r] = fmaf(xv, wv[d][i], acc[d][r]);
-        }
-      }
-    }
+  for (int r = 0; r < MT; ++r) xr[r] = m0 + r < m_hi ? (a.x_rows ? a.x_rows[m0 + r] : m0 + r) : -1;
+  for (int k0 = lane * 8; k0 < a.K; k0 += 64 * 8) {
+    float wv[DUAL ? 2 : 1][8];
+    load8<TW>(w + (int64_t)n * a.K + k0, a.K - k0, w_vec, wv[0]);
+    if (DUAL) load8<TW>(w2 + (int64_t)n * a.K + k0, a.K - k0, w_vec, wv[DUAL ? 1 : 0]);
 #pragma unroll
     for (int r = 0; r < MT; ++r) {
-      float v = wave_sum(acc[0][r]);
-      if (DUAL) v = silu_f(v) * wave_sum(acc[1][r]);
-      if (lane == 0 && xr[r] >= 0) {
-        const int64_t yrow = a.y_rows ? a.y_rows[m0 + r] : m0 + r;
-        a.y[yrow * a.ldy + n] = v * a.alpha;
-      }
+      if (xr[r] < 0) continue;
+      float xv[8];
+      load8<float>(a.x + xr[r] * a.ldx + k0, a.K - k0, x_vec, xv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int d = 0; d < (DUAL ? 2 : 1); ++d) acc[d][r] = fmaf(xv[i], wv[d][i], acc[d][r]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < MT; ++r) {
+    float v = wave_sum(acc[0][r]);
+    if (DUAL) v = silu_f(v) * wave_sum(acc[DUAL ? 1 : 0][r]);
+    if (lane == 0 && xr[r] >= 0) {
+      const int64_t yrow = a.y_rows ? a.y_rows[m0 + r] : m0 + r;
+      a.y[yrow * a.ldy + n] = v * a.alpha;
     }
   }
 }
@@ -277,10 +304,14 @@ __global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
 template <typename TW, bool DUAL>
 static int launch_any(const GemmAnyArgs& a, int groups, int rows_per_group_max, int mode, hipStream_t st) {
   // mode 0: product (MFMA for bf16 weights, the row kernel for few rows); 1: exact (FMA chains / row kernel, x unrounded)
-  if (rows_per_group_max <= 8) {
-    const dim3 grid((a.N + 3) / 4, 1, groups);
-    if (rows_per_group_max <= 1) hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 1, DUAL>), grid, dim3(256), 0, st, a);
-    else if (rows_per_group_max <= 4) hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 4, DUAL>), grid, dim3(256), 0, st, a);
+  // few rows (per group): the weight-streaming row kernel.  Also the exact mode up to 64 rows: a router's few output
+  // features would make one tile of the FMA kernel walk all of K alone
+  const bool few = rows_per_group_max <= 8 || (mode == 1 && rows_per_group_max <= 64);
+  if (few) {
+    const int mt = rows_per_group_max <= 1 ? 1 : rows_per_group_max <= 4 ? 4 : 8;
+    const dim3 grid((a.N + 3) / 4, (rows_per_group_max + mt - 1) / mt, groups);
+    if (mt == 1) hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 1, DUAL>), grid, dim3(256), 0, st, a);
+    else if (mt == 4) hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 4, DUAL>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((gemm_any_rows_kernel<TW, 8, DUAL>), grid, dim3(256), 0, st, a);
     return check_launch();
   }

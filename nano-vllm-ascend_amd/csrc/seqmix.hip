@@ -134,7 +134,8 @@ __global__ __launch_bounds__(256) void swa_prepare_kernel(float* __restrict__ pr
   }
 }
 
-// One wave per (row, head); lanes over keys for the scores, over value channels for the output.
+// The general form (any head sizes): one wave per (row, head); lanes over keys for the scores, over value channels for
+// the output, element-wise loads.
 template <typename TC, int VPL>  // VPL: value channels per lane (Dv <= 64 * VPL)
 __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restrict__ q, int64_t ldq,
                                                             const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
@@ -205,6 +206,168 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
       if (gate) o *= sigmoid_f(gate[(int64_t)row * ldg + h * Dv + d]);
       out[(int64_t)row * ldo + h * Dv + d] = o;
     }
+  }
+}
+
+// The product form: head sizes that are whole 16-byte pieces (D and Dv multiples of 8 for a bf16 cache, of 4 for fp32).
+// A wave takes RPW consecutive step rows of one head; rows of the same sequence (consecutive positions, windows that
+// differ by one key each) are handled TOGETHER: every K vector a lane loads is dotted with all of their queries, every
+// V vector multiplied into all of their accumulators, so a prompt's portion reads its keys and values RPW times less
+// often than row by row.  Scores: lane = key, the key's row in 16-byte loads.  Output: a V row is covered by LPR lanes
+// (16-byte piece each), 64 / LPR keys per pass, the key groups' partial sums added at the end.  Online softmax per row
+// with the usual guard for a chunk in which a row sees nothing yet.
+template <typename TC, int VEC>
+__device__ __forceinline__ void ld_vec(const TC* p, float (&v)[VEC]);
+template <>
+__device__ __forceinline__ void ld_vec<uint16_t, 8>(const uint16_t* p, float (&v)[8]) {
+  const u32x4 w = *reinterpret_cast<const u32x4*>(p);
+  v[0] = lo_bf(w[0]), v[1] = hi_bf(w[0]), v[2] = lo_bf(w[1]), v[3] = hi_bf(w[1]);
+  v[4] = lo_bf(w[2]), v[5] = hi_bf(w[2]), v[6] = lo_bf(w[3]), v[7] = hi_bf(w[3]);
+}
+template <>
+__device__ __forceinline__ void ld_vec<float, 4>(const float* p, float (&v)[4]) {
+  const float4 w = *reinterpret_cast<const float4*>(p);
+  v[0] = w.x, v[1] = w.y, v[2] = w.z, v[3] = w.w;
+}
+
+// SPLIT = 4 (single-row steps: decode): the four waves of a workgroup share ONE (row, head), take the window's 64-key
+// chunks in turn and merge their (max, sum, accumulator) triples through LDS - four times the waves in flight where a
+// step has only rows x heads units of work.
+template <typename TC, int VEC, int RPW, int SPLIT>
+__global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __restrict__ q, int64_t ldq,
+                                                                const TC* __restrict__ k_cache,
+                                                                const TC* __restrict__ v_cache,
+                                                                const int32_t* __restrict__ block_tables, int table_cols,
+                                                                const int32_t* __restrict__ cu_q,
+                                                                const int32_t* __restrict__ kv_lens, int n_seqs,
+                                                                int n_rows, int H, int G, int D, int Dv, int block_size,
+                                                                int window, float scale, int lpr_log2,
+                                                                const float* __restrict__ gate, int64_t ldg,
+                                                                float* __restrict__ out, int64_t ldo) {
+  static_assert(SPLIT == 1 || RPW == 1, "the split form is the single-row form");
+  extern __shared__ float smem[];  // per wave: q [RPW][D], p [RPW][64]; SPLIT > 1: then per wave {m, l, acc [Dv]}
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wid = SPLIT > 1 ? (int)blockIdx.x : (int)blockIdx.x * 4 + wave;
+  const int cw = SPLIT > 1 ? wave : 0;
+  const int n_groups = (n_rows + RPW - 1) / RPW;
+  if (wid >= n_groups * H) return;  // (SPLIT > 1: the whole workgroup)
+  const int rg = wid / H, h = wid % H;
+  float* qs = smem + wave * RPW * (D + 64);
+  float* ps = qs + RPW * D;
+  const int g = h / (H / G);
+  const float slope = exp2f(-8.f * (float)(h + 1) / (float)H);
+  const int lpr = 1 << lpr_log2, kg = lane >> lpr_log2, cg = lane & (lpr - 1), kpp = 64 >> lpr_log2;
+  const int group_end = min(rg * RPW + RPW, n_rows);
+  for (int first = rg * RPW; first < group_end;) {
+    const int s = seq_of_row(cu_q, n_seqs, first);
+    const int end = min(cu_q[s + 1], group_end), nr = end - first;
+    const int pos0 = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (first - cu_q[s]);
+    const int32_t* table = block_tables + (int64_t)s * table_cols;
+    __builtin_amdgcn_wave_barrier();
+    for (int r = 0; r < nr; ++r)
+      for (int d = lane; d < D; d += 64) qs[r * D + d] = q[(int64_t)(first + r) * ldq + h * D + d];
+    __builtin_amdgcn_wave_barrier();
+    const int lo = max(0, pos0 - window + 1), hi = pos0 + nr - 1;
+    float m[RPW], l[RPW], acc[RPW][VEC];
+#pragma unroll
+    for (int r = 0; r < RPW; ++r) {
+      m[r] = -INFINITY, l[r] = 0.f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[r][e] = 0.f;
+    }
+    for (int j0 = lo + 64 * cw; j0 <= hi; j0 += 64 * SPLIT) {
+      const int j = j0 + lane;
+      float dots[RPW];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) dots[r] = 0.f;
+      if (j <= hi) {
+        const int64_t blk = table[j / block_size];
+        const TC* kr = k_cache + ((blk * G + g) * block_size + j % block_size) * D;
+        for (int d0 = 0; d0 < D; d0 += VEC) {
+          float kv[VEC];
+          ld_vec<TC, VEC>(kr + d0, kv);
+#pragma unroll
+          for (int r = 0; r < RPW; ++r)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) dots[r] = fmaf(qs[r * D + d0 + e], kv[e], dots[r]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        const int pos = pos0 + r;
+        const bool vis = r < nr && j <= pos && j > pos - window;
+        const float sc = vis ? dots[r] * scale - slope * (float)(pos - j) : -INFINITY;
+        const float m_new = fmaxf(m[r], wave_max(sc));
+        const float p = vis ? expf(sc - m_new) : 0.f;
+        const float corr = m[r] == -INFINITY ? 0.f : expf(m[r] - m_new);
+        l[r] = l[r] * corr + wave_sum(p);
+        m[r] = m_new;
+        ps[r * 64 + lane] = p;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[r][e] *= corr;
+      }
+      __builtin_amdgcn_wave_barrier();
+      const int nk = min(64, hi - j0 + 1);
+      if (cg * VEC < Dv) {
+        for (int jj = kg; jj < nk; jj += kpp) {
+          const int jk = j0 + jj;
+          const int64_t blk = table[jk / block_size];
+          float vv[VEC];
+          ld_vec<TC, VEC>(v_cache + ((blk * G + g) * block_size + jk % block_size) * Dv + cg * VEC, vv);
+#pragma unroll
+          for (int r = 0; r < RPW; ++r) {
+            const float pj = ps[r * 64 + jj];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[r][e] = fmaf(pj, vv[e], acc[r][e]);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    for (int off = lpr; off < 64; off <<= 1)
+#pragma unroll
+      for (int r = 0; r < RPW; ++r)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[r][e] += __shfl_xor(acc[r][e], off);
+    if constexpr (SPLIT > 1) {
+      float* part = smem + 4 * RPW * (D + 64);  // [SPLIT][2 + Dv]
+      if (kg == 0 && cg * VEC < Dv)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) part[wave * (2 + Dv) + 2 + cg * VEC + e] = acc[0][e];
+      if (lane == 0) part[wave * (2 + Dv)] = m[0], part[wave * (2 + Dv) + 1] = l[0];
+      __syncthreads();
+      if (wave != 0) return;
+      float mm = -INFINITY;
+      for (int w2 = 0; w2 < SPLIT; ++w2) mm = fmaxf(mm, part[w2 * (2 + Dv)]);
+      float lsum = 0.f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) acc[0][e] = 0.f;
+      for (int w2 = 0; w2 < SPLIT; ++w2) {  // (a wave without a chunk: max -inf, weight 0)
+        const float mw = part[w2 * (2 + Dv)];
+        const float f = mw == -INFINITY ? 0.f : expf(mw - mm);
+        lsum = fmaf(part[w2 * (2 + Dv) + 1], f, lsum);
+        if (cg * VEC < Dv)
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[0][e] = fmaf(part[w2 * (2 + Dv) + 2 + cg * VEC + e], f, acc[0][e]);
+      }
+      l[0] = lsum;
+    }
+    if (kg == 0 && cg * VEC < Dv) {
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        if (r >= nr) continue;
+        const float inv = 1.f / l[r];
+        const int64_t row = first + r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const int d = cg * VEC + e;
+          float o = acc[r][e] * inv;
+          if (gate) o *= sigmoid_f(gate[row * ldg + h * Dv + d]);
+          out[row * ldo + h * Dv + d] = o;
+        }
+      }
+    }
+    first = end;
   }
 }
 
@@ -394,46 +557,106 @@ __global__ __launch_bounds__(256) void delta_finish_kernel(float* __restrict__ o
 // ---------------------------------------------------------------------------------------------------------------
 // sparse feed-forward: routing and combination
 // ---------------------------------------------------------------------------------------------------------------
-// One thread per token (n <= 512 router outputs, walked from global memory: the logits row is a few cache lines).
-__global__ __launch_bounds__(64) void route_grouped_kernel(const float* __restrict__ logits, int64_t ld,
-                                                           const float* __restrict__ correction, int T, int n, int top_k,
-                                                           int n_groups, int keep, int32_t* __restrict__ ids,
-                                                           float* __restrict__ wts) {
-  const int t = blockIdx.x * 64 + threadIdx.x;
+// One wave per token; a lane holds the outputs lane, lane + 64, ... (n <= 512: eight per lane).  Choice scores go through
+// LDS for the group maxima; groups and then outputs are picked by repeated arg-max over the wave (larger value first,
+// equal values: the lower index), NaN scores counting as 0.
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(v, off);
+    const int oi = __shfl_xor(idx, off);
+    if (ov > v || (ov == v && oi < idx)) v = ov, idx = oi;
+  }
+}
+
+__global__ __launch_bounds__(256) void route_grouped_kernel(const float* __restrict__ logits, int64_t ld,
+                                                            const float* __restrict__ correction, int T, int n, int top_k,
+                                                            int n_groups, int keep, int32_t* __restrict__ ids,
+                                                            float* __restrict__ wts) {
+  __shared__ float choice_s[4][512];
+  __shared__ int kept_s[4][512];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
   const float* z = logits + (int64_t)t * ld;
+  constexpr int EPL = 8;
+  const int big = 1 << 30;
+  float sc[EPL], ch[EPL];
   float mx = -INFINITY;
-  for (int e = 0; e < n; ++e) mx = fmaxf(mx, z[e]);
-  float sum = 0.f;
-  for (int e = 0; e < n; ++e) sum += expf(z[e] - mx);
-  const int per = n / n_groups;
-  // groups kept: `keep` times the best remaining group (score = its largest choice score; ties: the lower index)
-  uint64_t kept[8] = {};  // n_groups <= 512
-  for (int it = 0; it < keep; ++it) {
-    int best = -1;
-    float best_v = -INFINITY;
-    for (int gi = 0; gi < n_groups; ++gi) {
-      if (kept[gi >> 6] >> (gi & 63) & 1) continue;
-      float gv = -INFINITY;
-      for (int e = gi * per; e < (gi + 1) * per; ++e) gv = fmaxf(gv, expf(z[e] - mx) / sum + correction[e]);
-      if (best < 0 || gv > best_v) best = gi, best_v = gv;
-    }
-    kept[best >> 6] |= 1ull << (best & 63);
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    sc[i] = e < n ? z[e] : -INFINITY;
+    mx = fmaxf(mx, sc[i]);
   }
-  uint64_t taken[8] = {};  // n <= 512
-  for (int it = 0; it < top_k; ++it) {
-    int best = -1;
-    float best_v = -INFINITY, best_s = 0.f;
-    for (int e = 0; e < n; ++e) {
-      const int gi = e / per;
-      if (!(kept[gi >> 6] >> (gi & 63) & 1) || (taken[e >> 6] >> (e & 63) & 1)) continue;
-      const float sc = expf(z[e] - mx) / sum;
-      const float ch = sc + correction[e];
-      if (best < 0 || ch > best_v) best = e, best_v = ch, best_s = sc;
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    sc[i] = lane + 64 * i < n ? expf(sc[i] - mx) : 0.f;
+    sum += sc[i];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    sc[i] = sc[i] / sum;
+    if (!(sc[i] == sc[i])) sc[i] = 0.f;
+    ch[i] = e < n ? sc[i] + correction[e] : -INFINITY;
+    if (e < n) choice_s[wave][e] = ch[i];
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int per = n / n_groups;
+  float gsc[EPL];
+  unsigned g_taken = 0;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int gi = lane + 64 * i;
+    float gv = -INFINITY;
+    if (gi < n_groups) {
+      for (int e = gi * per; e < (gi + 1) * per; ++e) gv = fmaxf(gv, choice_s[wave][e]);
+      kept_s[wave][gi] = 0;
     }
-    taken[best >> 6] |= 1ull << (best & 63);
-    ids[(int64_t)t * top_k + it] = best;
-    wts[(int64_t)t * top_k + it] = best_s;
+    gsc[i] = gv;
+  }
+  for (int it = 0; it < keep; ++it) {
+    float bv = -INFINITY;
+    int bi = big;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int gi = lane + 64 * i;
+      if (gi < n_groups && !(g_taken >> i & 1) && (bi == big || gsc[i] > bv)) bv = gsc[i], bi = gi;
+    }
+    wave_argmax(bv, bi);
+    if ((bi & 63) == lane) {
+      g_taken |= 1u << (bi >> 6);
+      kept_s[wave][bi] = 1;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  unsigned taken = 0;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    if (e >= n || !kept_s[wave][e / per]) taken |= 1u << i;  // not eligible
+  }
+  for (int it = 0; it < top_k; ++it) {
+    float bv = -INFINITY;
+    int bi = big;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (!(taken >> i & 1) && (bi == big || ch[i] > bv)) bv = ch[i], bi = lane + 64 * i;
+    wave_argmax(bv, bi);
+    if ((bi & 63) == lane) {
+      const int i = bi >> 6;
+      taken |= 1u << i;
+      ids[(int64_t)t * top_k + it] = bi;
+      float w = 0.f;
+#pragma unroll
+      for (int i2 = 0; i2 < EPL; ++i2)
+        if (i2 == i) w = sc[i2];
+      wts[(int64_t)t * top_k + it] = w;
+    }
   }
 }
 
@@ -504,10 +727,30 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
                       const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
                       int block_size, int window, float scale, const float* gate, int64_t ldg, float* out, int64_t ldo,
                       hipStream_t st) {
-  const dim3 grid((rows * H + 3) / 4), block(256);
-  const size_t lds = 4 * (size_t)(D + 64) * sizeof(float);
   const TC* k = static_cast<const TC*>(kc);
   const TC* v = static_cast<const TC*>(vc);
+  constexpr int VEC = 16 / sizeof(TC);
+  if (D % VEC == 0 && Dv % VEC == 0 && Dv / VEC <= 64) {
+    int lpr_log2 = 0;
+    while ((1 << lpr_log2) * VEC < Dv) ++lpr_log2;
+    // rows == n_seqs: every sequence brings one row (a decode step): a wave per row; else four rows per wave
+    const int rpw = rows > n_seqs ? 4 : 1;
+    const size_t lds_v = (4 * (size_t)rpw * (D + 64) + (rpw == 1 ? 4 * (size_t)(2 + Dv) : 0)) * sizeof(float);
+    if (lds_v <= 48 * 1024) {
+      if (rpw == 4)
+        hipLaunchKernelGGL((swa_attention_vec_kernel<TC, VEC, 4, 1>), dim3((((rows + 3) / 4) * H + 3) / 4), dim3(256),
+                           lds_v, st, q, ldq, k, v, bt, cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window,
+                           scale, lpr_log2, gate, ldg, out, ldo);
+      else
+        hipLaunchKernelGGL((swa_attention_vec_kernel<TC, VEC, 1, 4>), dim3(rows * H), dim3(256), lds_v, st, q, ldq, k, v,
+                           bt, cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window, scale, lpr_log2, gate,
+                           ldg, out, ldo);
+      return check_launch();
+    }
+  }
+  const dim3 grid((rows * H + 3) / 4), block(256);
+  const size_t lds = 4 * (size_t)(D + 64) * sizeof(float);
+  if (lds > 48 * 1024) return MI_EUNSUPPORTED;
 #define MI_SWA(VPL)                                                                                                  \
   hipLaunchKernelGGL((swa_attention_kernel<TC, VPL>), grid, block, lds, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,     \
                      n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo)
@@ -599,7 +842,7 @@ extern "C" int mi_route_grouped(const float* logits, int64_t ld, const float* co
       top_k < 1 || top_k > keep * (n_outputs / n_groups))
     return MI_EUNSUPPORTED;
   if (n_tokens == 0) return MI_OK;
-  hipLaunchKernelGGL(route_grouped_kernel, dim3((n_tokens + 63) / 64), dim3(64), 0, S(stream), logits, ld, correction,
+  hipLaunchKernelGGL(route_grouped_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, S(stream), logits, ld, correction,
                      n_tokens, n_outputs, top_k, n_groups, keep, ids, weights);
   return check_launch();
 }

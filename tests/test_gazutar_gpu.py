@@ -40,6 +40,7 @@ def mixed_replay(request, mixed_model):
     ("attention", [with_mlp(attention(), None)]),
     ("attention_one_group", [with_mlp(attention(heads=4, kv_heads=4, dim=24, vdim=72, window=5), None)]),
     ("attention_gqa_all", [with_mlp(attention(heads=8, kv_heads=1, dim=16, vdim=8, window=64), None)]),
+    ("attention_odd_sizes", [with_mlp(attention(heads=2, kv_heads=1, dim=10, vdim=6, window=8), None)]),  # element-wise loads
     ("value_mixing", [with_mlp(attention(v_mix=True), None), with_mlp(attention(v_mix=True, window=30), None),
                       with_mlp(attention(v_mix=True, window=3), None)]),
     ("delta", [with_mlp(delta(), None)]),
