@@ -3,10 +3,12 @@
 // expert-sorted rows (one launch for all experts of a sparse feed-forward, SwiGLU optionally in the epilogue).
 //
 // These serve the model families whose residual stream, norms and recurrences are kept in 32-bit floats and whose
-// widths are not the fragment-native kernels' (csrc/gemm_skinny*.hpp, gemm_tile.hip): three kernels,
+// widths are not the fragment-native kernels' (csrc/gemm_skinny*.hpp, gemm_tile.hip): four kernels,
 //
 //   gemm_any_mfma_kernel   bf16 weights: 64 x 64 output tile per 4-wave workgroup, x rounded to bf16 on its way into
 //                          LDS, v_mfma_f32_16x16x32_bf16, edges zero-filled by guarded loads
+//   gemm_any_skinny_kernel bf16 weights, up to 64 rows per tile (decode batches, a decode step's experts): 16 features per
+//                          workgroup, the waves split K, fragments straight from memory
 //   gemm_any_fma_kernel    true 32-bit: fp32 (or bf16, widened exactly) weights, x NOT rounded, plain FMA chains in k
 //                          order - the float32 serving mode, and the routers of sparse feed-forwards in either mode
 //   gemm_any_rows_kernel   M <= 8 rows (decode): one wave per output feature streams its weight row once, lanes
@@ -251,6 +253,108 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// up to 64 rows per tile (decode batches, a decode step's experts): 16 output features per workgroup, so that even a
+// 1024-feature projection spreads over 64 workgroups; the four waves take the K steps of 32 in turn (together they read
+// 256 contiguous bytes of every weight row per round), operands go from memory straight into MFMA fragments - no LDS
+// staging, no barrier inside the K loop - and the waves' accumulators are added in wave order through LDS at the end.
+// ---------------------------------------------------------------------------------------------------------------
+template <bool DUAL, int MF>  // MF fragments of 16 rows
+__global__ __launch_bounds__(256) void gemm_any_skinny_kernel(GemmAnyArgs a) {
+  __shared__ __attribute__((aligned(16))) float red[3][DUAL ? 2 : 1][MF][64][4];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  int m_lo = 0, m_hi = a.M;
+  const uint16_t* w = static_cast<const uint16_t*>(a.w);
+  const uint16_t* w2 = static_cast<const uint16_t*>(a.w2);
+  if (a.group_offsets) {
+    m_lo = a.group_offsets[blockIdx.z];
+    m_hi = a.group_offsets[blockIdx.z + 1];
+    w += (int64_t)blockIdx.z * a.N * a.K;
+    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
+  }
+  const int m0 = m_lo + blockIdx.y * 16 * MF;
+  if (m0 >= m_hi) return;
+  const int n0 = blockIdx.x * 16;
+  const int fr = lane & 15, kk = (lane >> 4) * 8;
+  const int wrow = n0 + fr < a.N ? n0 + fr : -1;
+  int64_t xrow[MF];
+#pragma unroll
+  for (int f = 0; f < MF; ++f) {
+    const int m = m0 + f * 16 + fr;
+    xrow[f] = m < m_hi ? (a.x_rows ? a.x_rows[m] : m) : -1;
+  }
+  const bool w_vec = (a.K % 8 == 0) && dev_aligned16(a.w) && (!DUAL || dev_aligned16(a.w2));
+  const bool x_vec = (a.ldx % 4 == 0) && dev_aligned16(a.x);
+  f32x4 acc[DUAL ? 2 : 1][MF];
+#pragma unroll
+  for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+    for (int f = 0; f < MF; ++f) acc[d][f] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = wave * 32; k0 < a.K; k0 += 4 * 32) {
+    const int k = k0 + kk;
+    bf16x8 wf[DUAL ? 2 : 1];
+#pragma unroll
+    for (int d = 0; d < (DUAL ? 2 : 1); ++d) {
+      const uint16_t* wp = (d ? w2 : w) + (int64_t)wrow * a.K + k;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (wrow >= 0 && k < a.K) {
+        if (w_vec && k + 8 <= a.K) {
+          v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp));
+        } else {
+          uint16_t e[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) e[i] = k + i < a.K ? wp[i] : (uint16_t)0;
+          v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                    (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+        }
+      }
+      wf[d] = as_frag(v);
+    }
+#pragma unroll
+    for (int f = 0; f < MF; ++f) {
+      float xv[8];
+      if (xrow[f] >= 0) load8<float>(a.x + xrow[f] * a.ldx + k, a.K - k, x_vec, xv);
+      else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) xv[i] = 0.f;
+      }
+      const bf16x8 xf = as_frag(u32x4{pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])});
+#pragma unroll
+      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+        acc[d][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[d], xf, acc[d][f], 0, 0, 0);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+      for (int f = 0; f < MF; ++f) *reinterpret_cast<f32x4*>(red[wave - 1][d][f][lane]) = acc[d][f];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int ow = 0; ow < 3; ++ow)
+#pragma unroll
+    for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+#pragma unroll
+      for (int f = 0; f < MF; ++f) acc[d][f] += *reinterpret_cast<const f32x4*>(red[ow][d][f][lane]);
+  // a lane holds features n0 + (lane >> 4) * 4 + r of x row (lane & 15) of every fragment
+#pragma unroll
+  for (int f = 0; f < MF; ++f) {
+    const int m = m0 + f * 16 + fr;
+    if (m >= m_hi) continue;
+    const int64_t yrow = a.y_rows ? a.y_rows[m] : m;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + (lane >> 4) * 4 + r;
+      if (n >= a.N) continue;
+      float v = acc[0][f][r];
+      if (DUAL) v = silu_f(v) * acc[DUAL ? 1 : 0][f][r];
+      a.y[yrow * a.ldy + n] = v * a.alpha;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // few rows: one wave per output feature and batch of MT rows (blockIdx.y); the lanes take K in pieces of 8, ascending,
 // 16-byte loads where the operands allow it, then a butterfly over the lanes
 // ---------------------------------------------------------------------------------------------------------------
@@ -317,6 +421,17 @@ static int launch_any(const GemmAnyArgs& a, int groups, int rows_per_group_max, 
   }
   const dim3 grid((a.N + 63) / 64, (rows_per_group_max + 63) / 64, groups);
   if constexpr (sizeof(TW) == 2) {
+    if (mode == 0 && (rows_per_group_max <= 64 || (groups > 1 && rows_per_group_max <= 8 * groups))) {
+      // decode-sized: 16-feature workgroups (grouped: tiles of 32 rows, an expert's few rows fill the first)
+      if (groups > 1 || rows_per_group_max <= 32) {
+        const dim3 g2((a.N + 15) / 16, (rows_per_group_max + 31) / 32, groups);
+        hipLaunchKernelGGL((gemm_any_skinny_kernel<DUAL, 2>), g2, dim3(256), 0, st, a);
+      } else {
+        const dim3 g4((a.N + 15) / 16, 1, groups);
+        hipLaunchKernelGGL((gemm_any_skinny_kernel<DUAL, 4>), g4, dim3(256), 0, st, a);
+      }
+      return check_launch();
+    }
     if (mode == 0) {
       hipLaunchKernelGGL((gemm_any_mfma_kernel<DUAL>), grid, dim3(256), 0, st, a);
       return check_launch();
