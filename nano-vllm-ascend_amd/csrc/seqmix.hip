@@ -289,7 +289,13 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
 #pragma unroll
           for (int r = 0; r < RPW; ++r)
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) dots[r] = fmaf(qs[r * D + d0 + e], kv[e], dots[r]);
+            for (int e4 = 0; e4 < VEC; e4 += 4) {  // (D is a multiple of VEC: 16-byte LDS reads, the same address in every lane)
+              const float4 qv = *reinterpret_cast<const float4*>(qs + r * D + d0 + e4);
+              dots[r] = fmaf(qv.x, kv[e4], dots[r]);
+              dots[r] = fmaf(qv.y, kv[e4 + 1], dots[r]);
+              dots[r] = fmaf(qv.z, kv[e4 + 2], dots[r]);
+              dots[r] = fmaf(qv.w, kv[e4 + 3], dots[r]);
+            }
         }
       }
 #pragma unroll
@@ -504,19 +510,19 @@ __global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restr
       const float4* g4 = reinterpret_cast<const float4*>(gs[t]);
       const float4* k4 = reinterpret_cast<const float4*>(ks[t]);
       const float4* q4 = reinterpret_cast<const float4*>(qs[t]);
-      float dot = 0.f;
+      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;  // (four chains instead of one: the wave has its SIMD to itself)
 #pragma unroll
       for (int jj = 0; jj < DR / 4; ++jj) {
         const float4 gv = g4[jj * 4 + r], kv = k4[jj * 4 + r];
         st[jj * 4 + 0] *= gv.x, st[jj * 4 + 1] *= gv.y, st[jj * 4 + 2] *= gv.z, st[jj * 4 + 3] *= gv.w;
-        dot = fmaf(st[jj * 4 + 0], kv.x, dot);
-        dot = fmaf(st[jj * 4 + 1], kv.y, dot);
-        dot = fmaf(st[jj * 4 + 2], kv.z, dot);
-        dot = fmaf(st[jj * 4 + 3], kv.w, dot);
+        d0 = fmaf(st[jj * 4 + 0], kv.x, d0);
+        d1 = fmaf(st[jj * 4 + 1], kv.y, d1);
+        d2 = fmaf(st[jj * 4 + 2], kv.z, d2);
+        d3 = fmaf(st[jj * 4 + 3], kv.w, d3);
       }
-      dot = xor_sum<2>(xor_sum<1>(dot));
+      const float dot = xor_sum<2>(xor_sum<1>((d0 + d1) + (d2 + d3)));
       const float u = bs[t] * (vs[t][col] - dot);
-      float o = 0.f;
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
       for (int jj = 0; jj < DR / 4; ++jj) {
         const float4 kv = k4[jj * 4 + r], qv = q4[jj * 4 + r];
@@ -524,12 +530,12 @@ __global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restr
         st[jj * 4 + 1] = fmaf(kv.y, u, st[jj * 4 + 1]);
         st[jj * 4 + 2] = fmaf(kv.z, u, st[jj * 4 + 2]);
         st[jj * 4 + 3] = fmaf(kv.w, u, st[jj * 4 + 3]);
-        o = fmaf(st[jj * 4 + 0], qv.x, o);
-        o = fmaf(st[jj * 4 + 1], qv.y, o);
-        o = fmaf(st[jj * 4 + 2], qv.z, o);
-        o = fmaf(st[jj * 4 + 3], qv.w, o);
+        o0 = fmaf(st[jj * 4 + 0], qv.x, o0);
+        o1 = fmaf(st[jj * 4 + 1], qv.y, o1);
+        o2 = fmaf(st[jj * 4 + 2], qv.z, o2);
+        o3 = fmaf(st[jj * 4 + 3], qv.w, o3);
       }
-      o = xor_sum<2>(xor_sum<1>(o));
+      const float o = xor_sum<2>(xor_sum<1>((o0 + o1) + (o2 + o3)));
       if (r == 0 && c < Dv) out[(int64_t)(r0 + c0 + t) * ldo + h * Dv + c] = o;
     }
   }
