@@ -58,6 +58,9 @@ class Config:
     dtype: str = "bfloat16"
     # recurrent-state slots (models whose sequences carry a state beside their K/V pages); 0: max_num_seqs
     num_state_slots: int = 0
+    # hybrid models: the scheduler cuts prompts into portions of at most max_num_batched_tokens rows per step and batches
+    # them with the running sequences' decoded tokens (Scheduler.schedule_rows); False: whole-prompt prefill steps
+    chunked_prefill: bool = False
     hybrid_state: bool = False  # derived: the model class keeps recurrent state per sequence (no prefix sharing)
 
     def __post_init__(self):
@@ -89,7 +92,7 @@ class Config:
         eos = getattr(text, "eos_token_id", None)
         if eos is not None:
             self.eos = eos[0] if isinstance(eos, (list, tuple)) else eos
-        assert self.max_num_batched_tokens >= self.max_model_len
+        assert self.max_num_batched_tokens >= self.max_model_len or (self.chunked_prefill and self.hybrid_state)
 
     @property
     def use_graphs(self) -> bool:

@@ -236,6 +236,8 @@ class LLMEngine:
         if self._inflight_prefill is not None:
             queued, self._inflight_prefill = self._inflight_prefill, None
             return self._step_prefill(*queued)
+        if self.config.hybrid_state and self.config.chunked_prefill:
+            return self._step_rows()
         seqs, is_prefill = self.scheduler.schedule()
         if self.lookahead and not is_prefill and seqs and self.model_runner.can_launch_decode(len(seqs)):
             return self._step_lookahead(self.model_runner.call("launch_decode", seqs), seqs, set())
@@ -253,6 +255,21 @@ class LLMEngine:
                    for s in seqs if s.is_finished]
         num_tokens = sum(len(s) for s in seqs) if is_prefill else -len(seqs)
         return outputs, num_tokens
+
+    def _step_rows(self):
+        """Hybrid models with chunked prefill: the scheduler's step is a list of row runs - portions of prompts beside the
+        running sequences' decoded tokens; the runs that reach their sequence's end are sampled."""
+        runs = self.scheduler.schedule_rows()
+        if not runs:
+            return [], 0
+        done = [s for s, start, count in runs if start + count == len(s)]
+        prompt_rows = sum(count for s, start, count in runs if start < s.num_prompt_tokens)
+        token_ids = self.model_runner.call("run_row_step", runs)
+        self._stamp_first_tokens([s for s in done if s.num_completion_tokens == 0])
+        self.scheduler.postprocess(done, token_ids)
+        outputs = [(s.seq_id, s.completion_token_ids, s.num_prompt_tokens, s.num_cached_tokens)
+                   for s in done if s.is_finished]
+        return outputs, (prompt_rows if prompt_rows else -len(done))
 
     def _prefill_launchable(self, seqs) -> bool:
         runner = self.model_runner

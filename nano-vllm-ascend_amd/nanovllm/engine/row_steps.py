@@ -210,6 +210,34 @@ class RowSteps:
         ev.record()
         self._rg_events[b] = ev
 
+    @torch.inference_mode()
+    def run_row_step(self, runs) -> list[int]:
+        """One scheduler step of row runs (Scheduler.schedule_rows): portions and decoded tokens together; the runs that
+        reach their sequence's end get a token from the framework's sampler, in run order.  A step of single completing
+        rows is a decode step and replays its captured graph."""
+        done = [s for s, start, count in runs if start + count == len(s)]
+        if len(done) == len(runs) and all(count == 1 for _, _, count in runs):
+            return self.run_hybrid(done, False)
+        ends = np.cumsum([c for _, _, c in runs])
+        want = [int(e) - 1 for e, (s, start, count) in zip(ends, runs) if start + count == len(s)]
+        logits = self.run_rows(runs, want)
+        if not done:
+            torch.cuda.current_stream().synchronize()
+            return []
+        self.last_logits = logits
+        return self._sample_rows(logits, done)
+
+    def _sample_rows(self, logits, seqs) -> list[int]:
+        real = len(seqs)
+        temps = torch.tensor([0.0 if s.greedy else s.temperature for s in seqs], dtype=torch.float32).to(self.device)
+        # the sampler reads bf16 logits in rows of a multiple of 8 elements (layers/sampler.py)
+        vocab = logits.shape[1]
+        rounded = torch.empty((real, -(-vocab // 8) * 8), dtype=torch.bfloat16, device=self.device)[:, :vocab]
+        rounded.copy_(logits)
+        self.sampler(rounded, temps, out=self.tokens_dev[:real])
+        return self.tokens_dev[:real].tolist()
+
+    @torch.inference_mode()
     def run_hybrid(self, seqs, is_prefill: bool) -> list[int]:
         """ModelRunner.run for a hybrid model: the scheduler's prefill step (whole prompts; a preempted sequence comes back
         with its completion tokens and is recomputed from position 0, its state from zero) or decode step as row runs,
@@ -227,10 +255,4 @@ class RowSteps:
             runs = [(s, 0, len(s)) if is_prefill else (s, len(s) - 1, 1) for s in seqs]
             logits = self.run_rows(runs)
         self.last_logits = logits
-        temps = torch.tensor([0.0 if s.greedy else s.temperature for s in seqs], dtype=torch.float32).to(self.device)
-        # the sampler reads bf16 logits in rows of a multiple of 8 elements (layers/sampler.py)
-        vocab = logits.shape[1]
-        rounded = torch.empty((real, -(-vocab // 8) * 8), dtype=torch.bfloat16, device=self.device)[:, :vocab]
-        rounded.copy_(logits)
-        self.sampler(rounded, temps, out=self.tokens_dev[:real])
-        return self.tokens_dev[:real].tolist()
+        return self._sample_rows(logits, seqs)

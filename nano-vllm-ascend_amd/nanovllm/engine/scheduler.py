@@ -129,6 +129,54 @@ class Scheduler:
         seq.extend_tokens(token_ids)
         self.block_manager.extend(seq, len(seq))
 
+    def schedule_rows(self) -> list[tuple[Sequence, int, int]]:
+        """Hybrid models with chunked prefill: ONE step of row runs (sequence, start, count) - every running sequence's
+        next rows (its decoded token, or the next portion of its prompt), then, while the step's token budget, the
+        sequence count and the state slots last, first portions of waiting prompts.  Pages are taken as rows are
+        scheduled; when they run out the sequences at the right end of `running` are preempted as in `_pick_decode`
+        (a preempted sequence starts over at position 0)."""
+        assert self.state_slots is not None
+        bm, budget, runs, kept = self.block_manager, self.max_num_batched_tokens, [], []
+        while self.running:
+            seq = self.running.popleft()
+            n = min(len(seq) - seq.num_computed_tokens, budget)
+            if n <= 0 or len(runs) >= self.max_num_seqs:
+                kept.append(seq)  # (not in this step: the budget went to the sequences before it)
+                continue
+            evicted_self = False
+            while not bm.can_extend(seq, seq.num_computed_tokens + n):
+                if self.running:
+                    self.preempt(self.running.pop())
+                elif n > 1 and bm.can_extend(seq, seq.num_computed_tokens + 1):
+                    n = (len(seq.block_table) + len(bm.free_block_ids)) * bm.block_size - seq.num_computed_tokens
+                else:
+                    self.preempt(seq)
+                    evicted_self = True
+                    break
+            if evicted_self:
+                continue
+            bm.extend(seq, seq.num_computed_tokens + n)
+            runs.append((seq, seq.num_computed_tokens, n))
+            kept.append(seq)
+            budget -= n
+        self.running.extend(kept)
+        while (self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and len(runs) < self.max_num_seqs
+               and self.state_slots.free):
+            seq = self.waiting[0]
+            n = min(len(seq), budget)
+            if not bm.can_extend(seq, n):
+                break
+            self.waiting.popleft()
+            self.state_slots.acquire(seq)
+            seq.num_computed_tokens = 0
+            seq.table_gen += 1
+            seq.status = SequenceStatus.RUNNING
+            bm.extend(seq, n)
+            self.running.append(seq)
+            runs.append((seq, 0, n))
+            budget -= n
+        return runs
+
     def finish(self, seq: Sequence) -> None:
         """A sequence fed in portions is over: pages and slot go back."""
         self.free_seq(seq, FinishReason.LENGTH)

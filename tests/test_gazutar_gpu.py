@@ -326,6 +326,30 @@ def test_captured_decode_steps_equal_eager(mixed_model):
     assert rel_err(logits[1], logits[0]) <= CUT_BAR
 
 
+def test_engine_chunked_prefill_equals_whole_prompts(mixed_model):
+    """Config.chunked_prefill: the engine's own scheduler cuts prompts into portions (24 rows per step here) and batches
+    them with the other requests' decoded tokens; the generated tokens are those of whole-prompt prefill steps."""
+    from nanovllm import LLM, SamplingParams
+
+    cfg, w, d = mixed_model
+    prompts = [tokens_of(n, cfg["vocab"], 90 + n) for n in (70, 9, 41, 3, 26)]
+    sp = SamplingParams(max_tokens=9, greedy=True, ignore_eos=True)
+    runs = []
+    for kw in (dict(max_num_batched_tokens=128), dict(max_num_batched_tokens=24, chunked_prefill=True)):
+        llm = LLM(d, dtype="float32", kvcache_block_size=16, num_kvcache_blocks=40, max_num_seqs=3, max_model_len=128,
+                  warmup=False, **kw)
+        try:
+            runs.append([o["token_ids"] for o in llm.generate(prompts, sp, use_tqdm=False)])
+        finally:
+            llm.exit()
+    assert runs[0] == runs[1]
+    for prompt, gen in zip(prompts, runs[1]):
+        logits = expected(cfg, w, prompt + gen)
+        for i, tok in enumerate(gen):
+            row = logits[len(prompt) - 1 + i]
+            assert row.max() - row[tok] <= 0.06, (i, tok, int(row.argmax()))
+
+
 def test_preempted_request_is_recomputed(mixed_model):
     """So few pages that a running request is preempted: it gives its pages and slot back, comes back with its completion
     tokens and is recomputed from position 0 - the tokens are the ones it gets with room for everybody."""

@@ -117,3 +117,56 @@ def test_scheduler_steps_take_and_release_slots():
     picked, is_prefill = s.schedule()       # 33rd token: a page is needed - the last sequence is preempted
     assert not is_prefill and picked == [seqs[0]] and seqs[1].state_slot == -1 and not seqs[1].block_table
     assert s.waiting[0] is seqs[1] and seqs[0].state_slot == 0
+
+
+def test_row_scheduling_cuts_prompts_and_batches_decodes():
+    """schedule_rows(): a token budget of 32 rows per step - a long prompt goes in portions, the next prompt joins the step
+    that has budget left, a decoded token rides beside a portion, the third request waits for a slot."""
+    from nanovllm.engine.sequence import Sequence
+
+    s = _sched(pages=12, slots=2)
+    s.max_num_batched_tokens = 32
+    a, b, c = (Sequence([7] * n, block_size=16) for n in (50, 10, 5))
+    for q in (a, b, c):
+        q.max_tokens, q.ignore_eos = 3, True
+        s.add(q)
+
+    def step():
+        runs = s.schedule_rows()
+        done = [q for q, start, count in runs if start + count == len(q)]
+        for q, start, count in runs:
+            q.num_computed_tokens = start + count        # what the runner does
+        s.postprocess(done, [9] * len(done))
+        return [(q.seq_id - a.seq_id, start, count) for q, start, count in runs]
+
+    assert step() == [(0, 0, 32)]
+    assert step() == [(0, 32, 18), (1, 0, 10)] and (a.state_slot, b.state_slot, c.state_slot) == (0, 1, -1)
+    assert step() == [(0, 50, 1), (1, 10, 1)]
+    assert step() == [(0, 51, 1), (1, 11, 1)]            # both reach max_tokens = 3 and leave
+    assert a.is_finished and b.is_finished and s.state_slots.free == [1, 0]
+    assert step() == [(2, 0, 5)] and c.state_slot == 0
+    assert len(a.block_table) == 0 and len(c.block_table) == 1
+
+
+def test_row_scheduling_preempts_from_the_right_when_pages_run_out():
+    from nanovllm.engine.sequence import Sequence
+
+    s = _sched(pages=4, slots=2)
+    s.max_num_batched_tokens = 64
+    a, b = Sequence([1] * 31, block_size=16), Sequence([2] * 30, block_size=16)
+    for q in (a, b):
+        q.max_tokens, q.ignore_eos = 8, True
+        s.add(q)
+    runs = s.schedule_rows()
+    assert [(start, count) for _, start, count in runs] == [(0, 31), (0, 30)]
+    for q, start, count in runs:
+        q.num_computed_tokens = start + count
+    s.postprocess([a, b], [9, 9])                        # 32 and 31 tokens: the four pages are full
+    runs = s.schedule_rows()                             # a's 33rd token needs a fifth page: b goes
+    assert [(q is a, start, count) for q, start, count in runs] == [(True, 31, 1)] or \
+        [(q is a, start, count) for q, start, count in runs] == [(True, 31, 1), (False, 30, 1)]
+    for q, start, count in runs:
+        q.num_computed_tokens = start + count
+    s.postprocess([q for q, _, _ in runs], [9] * len(runs))
+    runs = s.schedule_rows()
+    assert runs[0][0] is a and b.state_slot == -1 and s.waiting[0] is b and not b.block_table
