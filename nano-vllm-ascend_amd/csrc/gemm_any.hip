@@ -142,15 +142,17 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// MFMA kernel (bf16 weights): 64 x 64 tile, 4 waves as 2 x 2, each wave 32 x 32 = 2 x 2 fragments of 16 x 16,
+// MFMA kernel (bf16 weights): 4 waves as 2 x 2, each FM x FN fragments of 16 x 16 - a 64 x 64 tile, or 128 x 128
+// (SwiGLU: 128 x 64) for prefill-sized launches, where every LDS fragment feeds four MFMAs instead of two;
 // K in steps of 64 (a weight row's piece = one 128-byte line).  LDS holds the tile's x rows and weight rows as bf16
 // [64][64 + 8].
 // ---------------------------------------------------------------------------------------------------------------
-template <bool DUAL>
+template <bool DUAL, int FM, int FN>  // a wave's tile: FM x FN fragments of 16 x 16; the workgroup's: 2 x 2 waves
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
-  constexpr int BM = 64, BN = 64, BK = 64, LD = BK + 8;
+  constexpr int BM = 32 * FM, BN = 32 * FN, BK = 64, LD = BK + 8;
+  constexpr int ND = DUAL ? 2 : 1;
   __shared__ __attribute__((aligned(16))) uint16_t As[BM][LD];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[DUAL ? 2 : 1][BN][LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[ND][BN][LD];
   const int tid = threadIdx.x;
   int m_lo = 0, m_hi = a.M;
   const uint16_t* w = static_cast<const uint16_t*>(a.w);
@@ -164,91 +166,112 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
   const int m0 = m_lo + blockIdx.y * BM;
   if (m0 >= m_hi) return;
   const int n0 = blockIdx.x * BN;
-  const int lr = tid >> 2, lk = (tid & 3) * 16;  // this thread stages 16 consecutive k of one row: a row's 64 k = one 128-byte line of weights
-  int64_t xrow = -1;
-  if (m0 + lr < m_hi) xrow = a.x_rows ? a.x_rows[m0 + lr] : m0 + lr;
-  const int wrow = n0 + lr < a.N ? n0 + lr : -1;
+  // staging: a thread takes 16 consecutive k of one row (a row's 64 k = one 128-byte line of weights), 64 rows per pass
+  const int lr = tid >> 2, lk = (tid & 3) * 16;
+  int64_t xrow[BM / 64];
+  int wrow[BN / 64];
+#pragma unroll
+  for (int p = 0; p < BM / 64; ++p) {
+    const int m = m0 + p * 64 + lr;
+    xrow[p] = m < m_hi ? (a.x_rows ? a.x_rows[m] : m) : -1;
+  }
+#pragma unroll
+  for (int p = 0; p < BN / 64; ++p) wrow[p] = n0 + p * 64 + lr < a.N ? n0 + p * 64 + lr : -1;
   const bool w_vec = (a.K % 8 == 0) && dev_aligned16(a.w) && (!DUAL || dev_aligned16(a.w2));
   const bool x_vec = (a.ldx % 4 == 0) && dev_aligned16(a.x);
   const int wave = tid >> 6, lane = tid & 63;
-  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  const int wm = (wave >> 1) * 16 * FM, wn = (wave & 1) * 16 * FN;
   const int fr = lane & 15, fk = (lane >> 4) * 8;
-  f32x4 acc[DUAL ? 2 : 1][2][2];
+  f32x4 acc[ND][FM][FN];
 #pragma unroll
-  for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+  for (int d = 0; d < ND; ++d)
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[d][i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < FN; ++j) acc[d][i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < a.K; k0 += BK) {
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int k = k0 + lk + half * 8;
-      float xv[8];
-      if (xrow >= 0) load8<float>(a.x + xrow * a.ldx + k, a.K - k, x_vec, xv);
-      else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xv[i] = 0.f;
-      }
-      const u32x4 xp = {pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
-      *reinterpret_cast<u32x4*>(&As[lr][lk + half * 8]) = xp;
+      for (int p = 0; p < BM / 64; ++p) {
+        float xv[8];
+        if (xrow[p] >= 0) load8<float>(a.x + xrow[p] * a.ldx + k, a.K - k, x_vec, xv);
+        else {
 #pragma unroll
-      for (int d = 0; d < (DUAL ? 2 : 1); ++d) {
-        const uint16_t* wp = (d ? w2 : w) + (int64_t)wrow * a.K + k;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (wrow >= 0 && k < a.K) {
-          if (w_vec && k + 8 <= a.K) {
-            v = *reinterpret_cast<const u32x4*>(wp);
-          } else {
-            uint16_t e[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) e[i] = k + i < a.K ? wp[i] : (uint16_t)0;
-            v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
-                      (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
-          }
+          for (int i = 0; i < 8; ++i) xv[i] = 0.f;
         }
-        *reinterpret_cast<u32x4*>(&Bs[d][lr][lk + half * 8]) = v;
+        const u32x4 xp = {pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
+        *reinterpret_cast<u32x4*>(&As[p * 64 + lr][lk + half * 8]) = xp;
       }
+#pragma unroll
+      for (int d = 0; d < ND; ++d)
+#pragma unroll
+        for (int p = 0; p < BN / 64; ++p) {
+          const uint16_t* wp = (d ? w2 : w) + (int64_t)wrow[p] * a.K + k;
+          u32x4 v = {0u, 0u, 0u, 0u};
+          if (wrow[p] >= 0 && k < a.K) {
+            if (w_vec && k + 8 <= a.K) {
+              v = *reinterpret_cast<const u32x4*>(wp);
+            } else {
+              uint16_t e[8];
+#pragma unroll
+              for (int i = 0; i < 8; ++i) e[i] = k + i < a.K ? wp[i] : (uint16_t)0;
+              v = u32x4{(uint32_t)e[0] | ((uint32_t)e[1] << 16), (uint32_t)e[2] | ((uint32_t)e[3] << 16),
+                        (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
+            }
+          }
+          *reinterpret_cast<u32x4*>(&Bs[d][p * 64 + lr][lk + half * 8]) = v;
+        }
     }
     __syncthreads();
     // D[n][m] = sum_k W[n][k] X[m][k]: weights on the MFMA's row axis, so a lane's four results are four consecutive
     // FEATURES of one x row
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      bf16x8 af[2], bfr[DUAL ? 2 : 1][2];
+      bf16x8 af[FM], bfr[ND][FN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) af[i] = as_frag(*reinterpret_cast<const u32x4*>(&As[wm + i * 16 + fr][ks * 32 + fk]));
+      for (int i = 0; i < FM; ++i) af[i] = as_frag(*reinterpret_cast<const u32x4*>(&As[wm + i * 16 + fr][ks * 32 + fk]));
 #pragma unroll
-      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+      for (int d = 0; d < ND; ++d)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < FN; ++j)
           bfr[d][j] = as_frag(*reinterpret_cast<const u32x4*>(&Bs[d][wn + j * 16 + fr][ks * 32 + fk]));
 #pragma unroll
-      for (int d = 0; d < (DUAL ? 2 : 1); ++d)
+      for (int d = 0; d < ND; ++d)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < FN; ++j)
             acc[d][i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[d][j], af[i], acc[d][i][j], 0, 0, 0);
     }
     __syncthreads();
   }
   // fragment (i, j): x row = wm + i*16 + (lane & 15), features wn + j*16 + (lane >> 4) * 4 + r
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < FM; ++i) {
     const int m = m0 + wm + i * 16 + (lane & 15);
     if (m >= m_hi) continue;
     const int64_t yrow = a.y_rows ? a.y_rows[m] : m;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < FN; ++j) {
+      const int n = n0 + wn + j * 16 + (lane >> 4) * 4;
+      float v[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int n = n0 + wn + j * 16 + (lane >> 4) * 4 + r;
-        if (n >= a.N) continue;
-        float v = acc[0][i][j][r];
-        if (DUAL) v = silu_f(v) * acc[DUAL ? 1 : 0][i][j][r];
-        a.y[yrow * a.ldy + n] = v * a.alpha;
+        v[r] = acc[0][i][j][r];
+        if (DUAL) v[r] = silu_f(v[r]) * acc[ND - 1][i][j][r];
+        v[r] *= a.alpha;
       }
+      float* yp = a.y + yrow * a.ldy + n;
+      if (n + 4 <= a.N && (a.ldy % 4 == 0) && dev_aligned16(a.y)) {
+        *reinterpret_cast<float4*>(yp) = float4{v[0], v[1], v[2], v[3]};
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < a.N) yp[r] = v[r];
+      }
+    }
   }
 }
 
@@ -421,6 +444,16 @@ static int launch_any(const GemmAnyArgs& a, int groups, int rows_per_group_max, 
   }
   const dim3 grid((a.N + 63) / 64, (rows_per_group_max + 63) / 64, groups);
   if constexpr (sizeof(TW) == 2) {
+    if (mode == 0 && rows_per_group_max >= 512 && a.N >= 128) {  // prefill-sized: 128-row tiles, 128 (SwiGLU: 64) features
+      if (DUAL) {
+        hipLaunchKernelGGL((gemm_any_mfma_kernel<DUAL, 4, 2>), dim3((a.N + 63) / 64, (rows_per_group_max + 127) / 128, groups),
+                           dim3(256), 0, st, a);
+      } else {
+        hipLaunchKernelGGL((gemm_any_mfma_kernel<DUAL, 4, 4>), dim3((a.N + 127) / 128, (rows_per_group_max + 127) / 128, groups),
+                           dim3(256), 0, st, a);
+      }
+      return check_launch();
+    }
     if (mode == 0 && (rows_per_group_max <= 64 || (groups > 1 && rows_per_group_max <= 8 * groups))) {
       // decode-sized: 16-feature workgroups (grouped: tiles of 32 rows, an expert's few rows fill the first)
       if (groups > 1 || rows_per_group_max <= 32) {
@@ -433,7 +466,7 @@ static int launch_any(const GemmAnyArgs& a, int groups, int rows_per_group_max, 
       return check_launch();
     }
     if (mode == 0) {
-      hipLaunchKernelGGL((gemm_any_mfma_kernel<DUAL>), grid, dim3(256), 0, st, a);
+      hipLaunchKernelGGL((gemm_any_mfma_kernel<DUAL, 2, 2>), grid, dim3(256), 0, st, a);
       return check_launch();
     }
   }

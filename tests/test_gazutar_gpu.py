@@ -84,7 +84,8 @@ def test_router_choices_and_weights():
     assert (wts.sum(-1) < 0.999).any()       # not renormalised
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 5, 129), (8, 64, 64), (9, 65, 31), (200, 130, 200), (64, 64, 32)])
+@pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 5, 129), (8, 64, 64), (9, 65, 31), (200, 130, 200), (64, 64, 32),
+                                   (600, 200, 100), (513, 128, 64), (40, 300, 264)])
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 def test_gemm_any_shapes(M, N, K, wdtype):
     from nanovllm import ops
@@ -98,6 +99,35 @@ def test_gemm_any_shapes(M, N, K, wdtype):
         rounds_x = wdtype == torch.bfloat16 and not exact and M > 8
         tol = 2e-2 if rounds_x else 1e-5
         assert (got - want).abs().max() <= tol * K ** 0.5, (exact, float((got - want).abs().max()))
+
+
+@pytest.mark.parametrize("rows,counts", [(700, [300, 0, 131, 269, 0]), (24, [3, 0, 9, 12, 0]), (6, [0, 6, 0, 0, 0]),
+                                          (130, [1, 128, 0, 1, 0])])
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dual", [False, True])
+def test_grouped_gemm_against_a_loop(rows, counts, wdtype, dual):
+    """The experts' grouped GEMM in each of its kernels (prefill-sized tiles, decode-sized tiles, row kernel): gathered input
+    rows, scattered output rows, empty groups, SwiGLU epilogue."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(rows)
+    E, N, K, T = len(counts), 88, 72, 50
+    x = torch.randn(T, K, generator=g)
+    w = (torch.randn(E, N, K, generator=g) * K ** -0.5).to(wdtype)
+    w2 = (torch.randn(E, N, K, generator=g) * K ** -0.5).to(wdtype) if dual else None
+    offsets = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32)
+    x_rows = torch.randint(0, T, (rows,), generator=g, dtype=torch.int32)
+    y_rows = torch.randperm(rows, generator=g).to(torch.int32)
+    got = ops.gemm_any_grouped(x.cuda(), x_rows.cuda(), w.cuda(), None if w2 is None else w2.cuda(), offsets.cuda(), rows,
+                               y_rows.cuda(), rows).cpu().double()
+    xr = x.bfloat16().double() if (wdtype == torch.bfloat16 and rows > 8) else x.double()
+    for e in range(E):
+        for p in range(int(offsets[e]), int(offsets[e + 1])):
+            h = xr[x_rows[p]]
+            want = h @ w[e].double().T
+            if dual:
+                want = torch.nn.functional.silu(want) * (h @ w2[e].double().T)
+            assert (got[y_rows[p]] - want).abs().max() <= 2e-4, (e, p)
 
 
 # ------------------------------------------------------------------------------------------------ cuts of one sequence
