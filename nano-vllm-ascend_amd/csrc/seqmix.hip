@@ -440,7 +440,7 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(const float* __r
 // rows of this step - lane r of the quad owns the channels (4 jj + r) * 4 + e, so that a quad's LDS reads of the row's
 // k / q / decay vectors are four consecutive 16-byte pieces and the two sums over the key channels end in two DPP steps
 // inside the quad.  Rows are prepared 16 at a time by all 256 threads (unit q and k, decay, sigmoid of beta, the value
-// columns) into LDS; between two preparations the walk needs no barrier.  The state is kept in memory in THREAD order
+// columns) into LDS, their inputs loaded one preparation ahead; between two preparations the walk needs no barrier.  The state is kept in memory in THREAD order
 // ([slot][head][column block][DR][256]: register ii of thread t at ii * 256 + t), read and written fully coalesced and
 // touched by nothing else.  The read-out is written raw; delta_finish_kernel applies the per-head RMS norm and gate.
 constexpr int kDeltaCols = 64, kDeltaRows = 16;
@@ -475,36 +475,56 @@ __global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restr
   const float decay_rate = expf(a_log[h]);
   const float q_scale = 1.f / sqrtf((float)D);
   const int pt = tid >> 4, ps = tid & 15;  // preparation: 16 lanes per row
+  // a row's raw q / k / decay inputs, value columns and beta input are LOADED one preparation ahead: the loads of rows
+  // c0 + 16 .. c0 + 31 are in flight while rows c0 .. c0 + 15 are walked
+  constexpr int PE = DR / 4;  // key channels per preparing lane (4 DR / 16)
+  float rq[PE], rk[PE], rd[PE], rv[kDeltaCols / 16], rb;
+  auto prep_load = [&](int c0) {
+    const bool live = c0 + pt < n;
+    const int64_t row = r0 + (live ? c0 + pt : 0);
+#pragma unroll
+    for (int m = 0; m < PE; ++m) {
+      const int i = ps + 16 * m;
+      const bool ok = live && i < D;
+      rq[m] = ok ? qkv[row * ld + q_off + kvh * D + i] : 0.f;
+      rk[m] = ok ? qkv[row * ld + k_off + kvh * D + i] : 0.f;
+      rd[m] = ok ? decay_pre[row * ld_decay + h * D + i] + dt_bias[h * D + i] : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < kDeltaCols / 16; ++m) {
+      const int cc = cb * kDeltaCols + ps + 16 * m;
+      rv[m] = (live && cc < Dv) ? qkv[row * ld + v_off + h * Dv + cc] : 0.f;
+    }
+    rb = live ? beta_pre[row * ld_beta + h] : 0.f;
+  };
+  prep_load(0);
   for (int c0 = 0; c0 < n; c0 += kDeltaRows) {
     __syncthreads();  // the previous rows' vectors have been consumed
     {
       const bool live = c0 + pt < n;
-      const int64_t row = r0 + c0 + (live ? pt : 0);
       float sq = 0.f, sk = 0.f;
-      for (int i = ps; i < D; i += 16) {
-        const float qv = qkv[row * ld + q_off + kvh * D + i], kv = qkv[row * ld + k_off + kvh * D + i];
-        sq = fmaf(qv, qv, sq);
-        sk = fmaf(kv, kv, sk);
+#pragma unroll
+      for (int m = 0; m < PE; ++m) {
+        sq = fmaf(rq[m], rq[m], sq);
+        sk = fmaf(rk[m], rk[m], sk);
       }
       sq = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>(sq))));
       sk = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>(sk))));
       const float nq = q_scale / sqrtf(sq + 1e-6f), nk = 1.f / sqrtf(sk + 1e-6f);
-      for (int i = ps; i < DP; i += 16) {
-        float qv = 0.f, kv = 0.f, gv = 0.f;
-        if (i < D && live) {
-          qv = qkv[row * ld + q_off + kvh * D + i] * nq;
-          kv = qkv[row * ld + k_off + kvh * D + i] * nk;
-          gv = expf(-decay_rate * softplus_f(decay_pre[row * ld_decay + h * D + i] + dt_bias[h * D + i]));
-        }
-        qs[pt][i] = qv, ks[pt][i] = kv, gs[pt][i] = gv;
+#pragma unroll
+      for (int m = 0; m < PE; ++m) {
+        const int i = ps + 16 * m;
+        const bool ok = live && i < D;
+        qs[pt][i] = rq[m] * nq;
+        ks[pt][i] = rk[m] * nk;
+        gs[pt][i] = ok ? expf(-decay_rate * softplus_f(rd[m])) : 0.f;
       }
-      for (int e = ps; e < kDeltaCols; e += 16) {
-        const int cc = cb * kDeltaCols + e;
-        vs[pt][e] = (live && cc < Dv) ? qkv[row * ld + v_off + h * Dv + cc] : 0.f;
-      }
-      if (ps == 0) bs[pt] = live ? sigmoid_f(beta_pre[row * ld_beta + h]) : 0.f;
+#pragma unroll
+      for (int m = 0; m < kDeltaCols / 16; ++m) vs[pt][ps + 16 * m] = rv[m];
+      if (ps == 0) bs[pt] = live ? sigmoid_f(rb) : 0.f;
     }
     __syncthreads();
+    if (c0 + kDeltaRows < n) prep_load(c0 + kDeltaRows);
     const int nt = min(kDeltaRows, n - c0);
     for (int t = 0; t < nt; ++t) {
       const float4* g4 = reinterpret_cast<const float4*>(gs[t]);
