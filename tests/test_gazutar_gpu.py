@@ -46,6 +46,7 @@ def mixed_replay(request, mixed_model):
     ("delta", [with_mlp(delta(), None)]),
     ("delta_wide_value", [with_mlp(delta(heads=3, kv_heads=1, dim=20, vdim=100, conv=2), None)]),
     ("delta_wide_key", [with_mlp(delta(heads=2, kv_heads=2, dim=130, vdim=24, conv=7), None)]),
+    ("delta_128", [with_mlp(delta(heads=2, kv_heads=1, dim=128, vdim=128, conv=4), None)]),
     ("delta_no_conv_memory", [with_mlp(delta(conv=1), None)]),
     ("sparse_ff", [with_mlp(attention(), moe())]),
     ("sparse_ff_no_identity_one_group", [with_mlp(delta(), moe(experts=7, identity=0, top=7, count=1, keep=1))]),
@@ -84,8 +85,23 @@ def test_router_choices_and_weights():
     assert (wts.sum(-1) < 0.999).any()       # not renormalised
 
 
+@pytest.mark.parametrize("n,experts,top,count,keep", [(130, 128, 6, 10, 3), (130, 126, 9, 65, 7), (512, 500, 8, 8, 2)])
+def test_router_many_outputs(n, experts, top, count, keep):
+    """More router outputs than lanes (several per lane), more groups than lanes."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(n + count)
+    z = torch.randn(40, n, generator=g) * 3
+    corr = torch.randn(n, generator=g) * 0.02
+    cfg = {"router": {"experts": experts, "identity": n - experts, "top": top, "groups": {"count": count, "keep": keep}}}
+    ids, wts = G.route(z.double(), {"router": torch.eye(n, dtype=torch.float64), "correction": corr.double()}, cfg)
+    got_ids, got_w = ops.route_grouped(z.cuda(), corr.cuda(), top, count, keep)
+    assert torch.equal(got_ids.cpu().long(), ids)
+    assert torch.allclose(got_w.cpu().double(), wts, atol=1e-6)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 5, 129), (8, 64, 64), (9, 65, 31), (200, 130, 200), (64, 64, 32),
-                                   (600, 200, 100), (513, 128, 64), (40, 300, 264)])
+                                   (600, 200, 100), (513, 128, 64), (40, 300, 264), (4, 50, 1100), (70, 33, 1100)])
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 def test_gemm_any_shapes(M, N, K, wdtype):
     from nanovllm import ops
@@ -167,6 +183,40 @@ def test_portions(mixed_model, mixed_replay, cuts):
     assert_close(got, expected(cfg, w, toks), dtype)
     if dtype == "float32":
         assert rel_err(got, r.feed("w", toks, [75])) <= CUT_BAR
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_windows_wider_than_a_chunk_of_keys(dtype):
+    """Windows of 70, 150 and 400 keys (the kernels take keys 64 at a time: several rounds of the running softmax, the
+    window's lower edge inside a round), head sizes 64 / 96 and 256 / 8, 330 tokens: whole, in portions, decoded."""
+    cfg = config([with_mlp(attention(heads=4, kv_heads=2, dim=64, vdim=96, window=150, scale=0.3, v_mix=True), None),
+                  with_mlp(attention(heads=2, kv_heads=2, dim=256, vdim=8, window=70, scale=0.2), None),
+                  with_mlp(attention(heads=4, kv_heads=2, dim=64, vdim=96, window=400, scale=0.3, v_mix=True), None)],
+                 width=96, vocab=61)
+    w = G.random_model(cfg, seed=21)
+    toks = tokens_of(330, 61, 8)
+    want = expected(cfg, w, toks)
+    r = Replay(write_model_dir(cfg, w), dtype, pages=48)
+    try:
+        assert_close(r.feed("a", toks, [330]), want, dtype)
+        assert_close(r.feed("b", toks, [100, 3, 64, 65, 2, 70]), want, dtype)     # then 26 single tokens
+        assert_close(r.feed("c", toks, [140] + [1] * 100 + [90]), want, dtype)
+    finally:
+        r.close()
+
+
+def test_wide_window_with_odd_head_sizes():
+    """The element-wise attention kernel (head sizes that are not whole 16-byte pieces) over several rounds of keys."""
+    cfg = config([with_mlp(attention(heads=3, kv_heads=1, dim=10, vdim=6, window=100, scale=0.4), None)], width=40, vocab=29)
+    w = G.random_model(cfg, seed=23)
+    toks = tokens_of(230, 29, 9)
+    want = expected(cfg, w, toks)
+    r = Replay(write_model_dir(cfg, w), "float32", pages=32)
+    try:
+        assert_close(r.feed("a", toks, [230]), want, "float32")
+        assert_close(r.feed("b", toks, [101, 2, 99] + [1] * 20 + [8]), want, "float32")
+    finally:
+        r.close()
 
 
 def test_long_decoding(mixed_model, mixed_replay):
