@@ -382,6 +382,26 @@ def test_greedy_generation_through_llm(mixed_model, dtype):
         llm.exit()
 
 
+def test_engine_with_default_start_up(mixed_model):
+    """LLM(model_dir) as a user calls it: warm-up generations, pages sized from free memory, captured decode steps."""
+    from nanovllm import LLM, SamplingParams
+
+    cfg, w, d = mixed_model
+    llm = LLM(d, kvcache_block_size=16, max_num_seqs=4, max_model_len=64, max_num_batched_tokens=256,
+              gpu_memory_utilization=0.05)
+    try:
+        assert llm.model_runner.row_graphs and llm.config.num_kvcache_blocks > 100
+        prompt = tokens_of(20, cfg["vocab"], 5)
+        out = llm.generate([prompt], SamplingParams(max_tokens=6, greedy=True, ignore_eos=True), use_tqdm=False)[0]
+        logits = expected(cfg, w, prompt + out["token_ids"])
+        for i, tok in enumerate(out["token_ids"]):
+            row = logits[len(prompt) - 1 + i]
+            assert row.max() - row[tok] <= 0.06
+        assert llm.ttft
+    finally:
+        llm.exit()
+
+
 def test_captured_decode_steps_equal_eager(mixed_model):
     """The engine's decode steps replay hipGraphs padded to a batch bucket (here 3 live requests in the bucket of 4, the
     padded row writing the spare state slot): same tokens and, for the real rows, the same logits as eager launches -
