@@ -189,7 +189,10 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
     for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j) acc[d][i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < a.K; k0 += BK) {
+  // the tile's operands travel memory -> registers -> LDS; the registers of K step k + 1 are loaded while step k's
+  // MFMAs run, so the global-memory latency is not paid between the two barriers
+  u32x4 xreg[2][BM / 64], wreg[ND][2][BN / 64];
+  auto fetch = [&](int k0) {
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int k = k0 + lk + half * 8;
@@ -201,8 +204,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
 #pragma unroll
           for (int i = 0; i < 8; ++i) xv[i] = 0.f;
         }
-        const u32x4 xp = {pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
-        *reinterpret_cast<u32x4*>(&As[p * 64 + lr][lk + half * 8]) = xp;
+        xreg[half][p] = u32x4{pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])};
       }
 #pragma unroll
       for (int d = 0; d < ND; ++d)
@@ -221,10 +223,23 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
                         (uint32_t)e[4] | ((uint32_t)e[5] << 16), (uint32_t)e[6] | ((uint32_t)e[7] << 16)};
             }
           }
-          *reinterpret_cast<u32x4*>(&Bs[d][p * 64 + lr][lk + half * 8]) = v;
+          wreg[d][half][p] = v;
         }
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int p = 0; p < BM / 64; ++p) *reinterpret_cast<u32x4*>(&As[p * 64 + lr][lk + half * 8]) = xreg[half][p];
+#pragma unroll
+      for (int d = 0; d < ND; ++d)
+#pragma unroll
+        for (int p = 0; p < BN / 64; ++p) *reinterpret_cast<u32x4*>(&Bs[d][p * 64 + lr][lk + half * 8]) = wreg[d][half][p];
+    }
     __syncthreads();
+    if (k0 + BK < a.K) fetch(k0 + BK);
     // D[n][m] = sum_k W[n][k] X[m][k]: weights on the MFMA's row axis, so a lane's four results are four consecutive
     // FEATURES of one x row
 #pragma unroll
