@@ -691,6 +691,8 @@ int mi_causal_conv_state(const float* x, int64_t ldx, int taps, float* state, co
 /* Floats of recurrent state one sequence slot holds for mi_channel_delta (the kernel's own thread-order layout), or
  * -1 when D is beyond the compiled kernels (D <= 256).  Host only. */
 int64_t mi_channel_delta_state_elems(int H, int D, int Dv);
+/* Floats of scratch mi_channel_delta needs for n_rows step rows (the rows' unit q / k, decays and betas).  Host only. */
+int64_t mi_channel_delta_workspace_elems(int n_rows, int H, int G, int D);
 /* Gated delta rule with a decay per (head, key channel); state [slots][mi_channel_delta_state_elems] fp32.  Per row and head h (q / k
  * head h / (H / G)): q, k <- unit vectors (x / sqrt(sum x^2 + 1e-6)), q / sqrt(D); g = exp(-exp(a_log[h]) *
  * softplus(decay_pre[row][h*D..] + dt_bias[h*D..])); beta = sigmoid(beta_pre[row][h]);
@@ -700,7 +702,7 @@ int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_o
                      int64_t ld_beta, const float* decay_pre, int64_t ld_decay, const float* dt_bias,
                      const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w, float* state,
                      const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int n_rows, int H,
-                     int G, int D, int Dv, float eps, float* out, int64_t ldo, mi_stream stream);
+                     int G, int D, int Dv, float eps, float* workspace, float* out, int64_t ldo, mi_stream stream);
 /* Router with expert groups: scores = softmax(logits) over n_outputs; choice = scores + correction; only the
  * `keep` of `n_groups` equal groups of neighbours with the largest best choice are eligible; ids = the top_k
  * eligible outputs by choice (descending), weights = their scores (not renormalised).  n_outputs <= 512. */

@@ -434,27 +434,55 @@ __global__ __launch_bounds__(256) void causal_conv_state_kernel(const float* __r
 // ---------------------------------------------------------------------------------------------------------------
 // gated delta rule, decay per head and key channel
 // ---------------------------------------------------------------------------------------------------------------
-// The columns of S (one per value channel) never exchange anything: S^T k, the rank-one update and S^T q are per-column
-// sums over the key channels.  One workgroup = 64 value columns of one (sequence, head); a column is held by FOUR lanes
-// (quad), each keeping DR of the (padded) 4 * DR key channels of it in registers for the whole walk over the sequence's
-// rows of this step - lane r of the quad owns the channels (4 jj + r) * 4 + e, so that a quad's LDS reads of the row's
-// k / q / decay vectors are four consecutive 16-byte pieces and the two sums over the key channels end in two DPP steps
-// inside the quad.  Rows are prepared 16 at a time by all 256 threads (unit q and k, decay, sigmoid of beta, the value
-// columns) into LDS, their inputs loaded one preparation ahead; between two preparations the walk needs no barrier.  The state is kept in memory in THREAD order
-// ([slot][head][column block][DR][256]: register ii of thread t at ii * 256 + t), read and written fully coalesced and
-// touched by nothing else.  The read-out is written raw; delta_finish_kernel applies the per-head RMS norm and gate.
-constexpr int kDeltaCols = 64, kDeltaRows = 16;
+// Three launches.  delta_prepare_kernel (parallel over rows): the row's unit q and k per q/k head, its decay vector and
+// beta per head - everything with a transcendental in it - into a workspace [rows][2 G D + H D + H].
+// channel_delta_kernel (the recurrence): the columns of S (one per value channel) never exchange anything: S^T k, the
+// rank-one update and S^T q are per-column sums over the key channels.  One workgroup = 32 value columns of one
+// (sequence, head); a column is held by FOUR lanes (a quad), each keeping DR of the (padded) 4 * DR key channels of it
+// in registers for the whole walk over the sequence's rows of this step - lane r of the quad owns the channels
+// (4 jj + r) * 4 + e, so that a quad's LDS reads of the row's k / q / decay vectors are four consecutive 16-byte pieces
+// and the two sums over the key channels end in two DPP steps inside the quad.  The prepared vectors of 16 rows at a
+// time are copied into LDS, loaded one batch ahead (in flight while the current batch is walked); between two batches
+// the walk needs no barrier.  The state is kept in memory in THREAD order ([slot][head][column block][DR][128]: register
+// ii of thread t at ii * 128 + t), read and written fully coalesced and touched by nothing else.
+// delta_finish_kernel: per-head RMS norm of the raw read-out, weight, sigmoid gate.
+constexpr int kDeltaCols = 32, kDeltaRows = 16, kDeltaThreads = 4 * kDeltaCols;
+
+// workspace row: [q G*D | k G*D | decay H*D | beta H]
+__global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restrict__ qkv, int64_t ld, int q_off, int k_off,
+                                                            const float* __restrict__ beta_pre, int64_t ld_beta,
+                                                            const float* __restrict__ decay_pre, int64_t ld_decay,
+                                                            const float* __restrict__ dt_bias,
+                                                            const float* __restrict__ a_log, int H, int G, int D,
+                                                            float* __restrict__ ws) {
+  const int64_t row = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* out = ws + row * (int64_t)(2 * G * D + H * D + H);
+  const float q_scale = 1.f / sqrtf((float)D);
+  for (int u = wave; u < 2 * G; u += 4) {  // (q | k, head): a wave each
+    const bool is_k = u >= G;
+    const float* src = qkv + row * ld + (is_k ? k_off + (u - G) * D : q_off + u * D);
+    float sq = 0.f;
+    for (int i = lane; i < D; i += 64) sq = fmaf(src[i], src[i], sq);
+    const float nrm = (is_k ? 1.f : q_scale) / sqrtf(wave_sum(sq) + 1e-6f);
+    for (int i = lane; i < D; i += 64) out[u * D + i] = src[i] * nrm;
+  }
+  for (int e = threadIdx.x; e < H * D; e += 256) {
+    const float rate = expf(a_log[e / D]);
+    out[2 * G * D + e] = expf(-rate * softplus_f(decay_pre[row * ld_decay + e] + dt_bias[e]));
+  }
+  for (int h = threadIdx.x; h < H; h += 256) out[2 * G * D + H * D + h] = sigmoid_f(beta_pre[row * ld_beta + h]);
+}
 
 template <int DR>
-__global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restrict__ qkv, int64_t ld, int q_off,
-                                                            int k_off, int v_off, const float* __restrict__ beta_pre,
-                                                            int64_t ld_beta, const float* __restrict__ decay_pre,
-                                                            int64_t ld_decay, const float* __restrict__ dt_bias,
-                                                            const float* __restrict__ a_log, float* __restrict__ state,
-                                                            const int32_t* __restrict__ cu_q,
-                                                            const int32_t* __restrict__ kv_lens,
-                                                            const int32_t* __restrict__ slot_ids, int H, int G, int D,
-                                                            int Dv, float* __restrict__ out, int64_t ldo) {
+__global__ __launch_bounds__(kDeltaThreads) void channel_delta_kernel(const float* __restrict__ qkv, int64_t ld, int v_off,
+                                                                      const float* __restrict__ ws,
+                                                                      float* __restrict__ state,
+                                                                      const int32_t* __restrict__ cu_q,
+                                                                      const int32_t* __restrict__ kv_lens,
+                                                                      const int32_t* __restrict__ slot_ids, int H, int G,
+                                                                      int D, int Dv, float* __restrict__ out,
+                                                                      int64_t ldo) {
   constexpr int DP = 4 * DR;  // padded key channels
   __shared__ __attribute__((aligned(16))) float qs[kDeltaRows][DP];
   __shared__ __attribute__((aligned(16))) float ks[kDeltaRows][DP];
@@ -468,63 +496,44 @@ __global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restr
   if (n == 0) return;
   const int start = kv_lens[s] - n;
   const int kvh = h / (H / G);
-  float* slot = state + (((int64_t)slot_ids[s] * H + h) * gridDim.z + cb) * DR * 256;
+  const int64_t ws_ld = 2 * G * D + H * D + H;
+  float* slot = state + (((int64_t)slot_ids[s] * H + h) * gridDim.z + cb) * DR * kDeltaThreads;
   float st[DR];
 #pragma unroll
-  for (int ii = 0; ii < DR; ++ii) st[ii] = start > 0 ? slot[ii * 256 + tid] : 0.f;
-  const float decay_rate = expf(a_log[h]);
-  const float q_scale = 1.f / sqrtf((float)D);
-  const int pt = tid >> 4, ps = tid & 15;  // preparation: 16 lanes per row
-  // a row's raw q / k / decay inputs, value columns and beta input are LOADED one preparation ahead: the loads of rows
-  // c0 + 16 .. c0 + 31 are in flight while rows c0 .. c0 + 15 are walked
-  constexpr int PE = DR / 4;  // key channels per preparing lane (4 DR / 16)
-  float rq[PE], rk[PE], rd[PE], rv[kDeltaCols / 16], rb;
-  auto prep_load = [&](int c0) {
+  for (int ii = 0; ii < DR; ++ii) st[ii] = start > 0 ? slot[ii * kDeltaThreads + tid] : 0.f;
+  // staging: 8 lanes per row copy the row's prepared vectors (zeros beyond D and beyond the step's rows)
+  const int pt = tid >> 3, ps = tid & 7;
+  constexpr int PE = DP / 8;
+  float rq[PE], rk[PE], rg[PE], rv[kDeltaCols / 8], rb;
+  auto fetch = [&](int c0) {
     const bool live = c0 + pt < n;
     const int64_t row = r0 + (live ? c0 + pt : 0);
+    const float* w = ws + row * ws_ld;
 #pragma unroll
     for (int m = 0; m < PE; ++m) {
-      const int i = ps + 16 * m;
+      const int i = ps + 8 * m;
       const bool ok = live && i < D;
-      rq[m] = ok ? qkv[row * ld + q_off + kvh * D + i] : 0.f;
-      rk[m] = ok ? qkv[row * ld + k_off + kvh * D + i] : 0.f;
-      rd[m] = ok ? decay_pre[row * ld_decay + h * D + i] + dt_bias[h * D + i] : 0.f;
+      rq[m] = ok ? w[kvh * D + i] : 0.f;
+      rk[m] = ok ? w[(G + kvh) * D + i] : 0.f;
+      rg[m] = ok ? w[2 * G * D + h * D + i] : 0.f;
     }
 #pragma unroll
-    for (int m = 0; m < kDeltaCols / 16; ++m) {
-      const int cc = cb * kDeltaCols + ps + 16 * m;
+    for (int m = 0; m < kDeltaCols / 8; ++m) {
+      const int cc = cb * kDeltaCols + ps + 8 * m;
       rv[m] = (live && cc < Dv) ? qkv[row * ld + v_off + h * Dv + cc] : 0.f;
     }
-    rb = live ? beta_pre[row * ld_beta + h] : 0.f;
+    rb = live ? w[2 * G * D + H * D + h] : 0.f;
   };
-  prep_load(0);
+  fetch(0);
   for (int c0 = 0; c0 < n; c0 += kDeltaRows) {
     __syncthreads();  // the previous rows' vectors have been consumed
-    {
-      const bool live = c0 + pt < n;
-      float sq = 0.f, sk = 0.f;
 #pragma unroll
-      for (int m = 0; m < PE; ++m) {
-        sq = fmaf(rq[m], rq[m], sq);
-        sk = fmaf(rk[m], rk[m], sk);
-      }
-      sq = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>(sq))));
-      sk = xor_sum<8>(xor_sum<4>(xor_sum<2>(xor_sum<1>(sk))));
-      const float nq = q_scale / sqrtf(sq + 1e-6f), nk = 1.f / sqrtf(sk + 1e-6f);
+    for (int m = 0; m < PE; ++m) qs[pt][ps + 8 * m] = rq[m], ks[pt][ps + 8 * m] = rk[m], gs[pt][ps + 8 * m] = rg[m];
 #pragma unroll
-      for (int m = 0; m < PE; ++m) {
-        const int i = ps + 16 * m;
-        const bool ok = live && i < D;
-        qs[pt][i] = rq[m] * nq;
-        ks[pt][i] = rk[m] * nk;
-        gs[pt][i] = ok ? expf(-decay_rate * softplus_f(rd[m])) : 0.f;
-      }
-#pragma unroll
-      for (int m = 0; m < kDeltaCols / 16; ++m) vs[pt][ps + 16 * m] = rv[m];
-      if (ps == 0) bs[pt] = live ? sigmoid_f(rb) : 0.f;
-    }
+    for (int m = 0; m < kDeltaCols / 8; ++m) vs[pt][ps + 8 * m] = rv[m];
+    if (ps == 0) bs[pt] = rb;
     __syncthreads();
-    if (c0 + kDeltaRows < n) prep_load(c0 + kDeltaRows);
+    if (c0 + kDeltaRows < n) fetch(c0 + kDeltaRows);
     const int nt = min(kDeltaRows, n - c0);
     for (int t = 0; t < nt; ++t) {
       const float4* g4 = reinterpret_cast<const float4*>(gs[t]);
@@ -560,7 +569,7 @@ __global__ __launch_bounds__(256) void channel_delta_kernel(const float* __restr
     }
   }
 #pragma unroll
-  for (int ii = 0; ii < DR; ++ii) slot[ii * 256 + tid] = st[ii];
+  for (int ii = 0; ii < DR; ++ii) slot[ii * kDeltaThreads + tid] = st[ii];
 }
 
 // out[row][h] <- out / rms(out over Dv) * norm_w * sigmoid(gate): one wave per (row, head), in place
@@ -831,26 +840,34 @@ static int delta_dr(int D) { return D <= 64 ? 16 : D <= 128 ? 32 : D <= 256 ? 64
 extern "C" int64_t mi_channel_delta_state_elems(int H, int D, int Dv) {
   const int dr = delta_dr(D);
   if (H < 1 || D < 1 || Dv < 1 || dr == 0) return -1;
-  return (int64_t)H * ((Dv + kDeltaCols - 1) / kDeltaCols) * dr * 256;
+  return (int64_t)H * ((Dv + kDeltaCols - 1) / kDeltaCols) * dr * kDeltaThreads;
+}
+
+extern "C" int64_t mi_channel_delta_workspace_elems(int n_rows, int H, int G, int D) {
+  if (n_rows < 0 || H < 1 || G < 1 || D < 1) return -1;
+  return (int64_t)n_rows * (2 * (int64_t)G * D + (int64_t)H * D + H);
 }
 
 extern "C" int mi_channel_delta(const float* qkv, int64_t ld, int q_off, int k_off, int v_off, const float* beta_pre,
                                 int64_t ld_beta, const float* decay_pre, int64_t ld_decay, const float* dt_bias,
                                 const float* a_log, const float* gate_pre, int64_t ld_gate, const float* norm_w,
                                 float* state, const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids,
-                                int n_seqs, int n_rows, int H, int G, int D, int Dv, float eps, float* out, int64_t ldo,
-                                mi_stream stream) {
+                                int n_seqs, int n_rows, int H, int G, int D, int Dv, float eps, float* workspace,
+                                float* out, int64_t ldo, mi_stream stream) {
   if (!qkv || !beta_pre || !decay_pre || !dt_bias || !a_log || !gate_pre || !norm_w || !state || !cu_q || !kv_lens ||
-      !slot_ids || !out || n_seqs < 1 || n_rows < 0)
+      !slot_ids || !out || !workspace || n_seqs < 1 || n_rows < 0)
     return MI_EINVAL;
   if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1) return MI_EINVAL;
   const int dr = delta_dr(D);
   if (dr == 0 || n_seqs > 65535) return MI_EUNSUPPORTED;
   if (n_rows == 0) return MI_OK;
-  const dim3 grid(n_seqs, H, (Dv + kDeltaCols - 1) / kDeltaCols), block(256);
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(n_rows), dim3(256), 0, S(stream), qkv, ld, q_off, k_off, beta_pre, ld_beta,
+                     decay_pre, ld_decay, dt_bias, a_log, H, G, D, workspace);
+  if (check_launch() != MI_OK) return MI_ELAUNCH;
+  const dim3 grid(n_seqs, H, (Dv + kDeltaCols - 1) / kDeltaCols), block(kDeltaThreads);
 #define MI_DELTA(DR)                                                                                                  \
-  hipLaunchKernelGGL((channel_delta_kernel<DR>), grid, block, 0, S(stream), qkv, ld, q_off, k_off, v_off, beta_pre,     \
-                     ld_beta, decay_pre, ld_decay, dt_bias, a_log, state, cu_q, kv_lens, slot_ids, H, G, D, Dv, out, ldo)
+  hipLaunchKernelGGL((channel_delta_kernel<DR>), grid, block, 0, S(stream), qkv, ld, v_off, workspace, state, cu_q,     \
+                     kv_lens, slot_ids, H, G, D, Dv, out, ldo)
   if (dr == 16) MI_DELTA(16);
   else if (dr == 32) MI_DELTA(32);
   else MI_DELTA(64);

@@ -176,8 +176,9 @@ _SIGNATURES = {
     "mi_causal_conv_silu": (c_int, [_p, c_int64, _p, c_int, _p, _p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p]),
     "mi_causal_conv_state": (c_int, [_p, c_int64, c_int, _p, _p, _p, _p, c_int, c_int, _p]),
     "mi_channel_delta_state_elems": (c_int64, [c_int, c_int, c_int]),
+    "mi_channel_delta_workspace_elems": (c_int64, [c_int, c_int, c_int, c_int]),
     "mi_channel_delta": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, c_int64, _p, c_int64, _p, _p, _p, c_int64, _p,
-                                 _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_int64, _p]),
+                                 _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, _p, c_int64, _p]),
     "mi_route_grouped": (c_int, [_p, c_int64, _p, c_int, c_int, c_int, c_int, c_int, _p, _p, _p]),
     "mi_moe_combine_f32": (c_int, [_p, _p, c_int64, _p, _p, c_int, c_int, c_int, c_int, _p, c_int64, _p]),
 }

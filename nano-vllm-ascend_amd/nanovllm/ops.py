@@ -1076,10 +1076,12 @@ def channel_delta(qkv, q_off: int, k_off: int, v_off: int, beta_pre, decay_pre, 
     assert beta_pre.shape == (rows, H) and decay_pre.shape == (rows, H * D) and gate_pre.shape == (rows, H * Dv)
     assert dt_bias.numel() == H * D and a_log.numel() == H and norm_w.numel() == Dv
     out = torch.empty((rows, H * Dv), dtype=_F32, device=qkv.device)
+    scratch = torch.empty(max(1, lib.mi_channel_delta_workspace_elems(rows, H, G, D)), dtype=_F32, device=qkv.device)
     check(lib.mi_channel_delta(ptr(qkv), qkv.stride(0), q_off, k_off, v_off, ptr(beta_pre), beta_pre.stride(0),
                                ptr(decay_pre), decay_pre.stride(0), ptr(dt_bias), ptr(a_log), ptr(gate_pre),
                                gate_pre.stride(0), ptr(norm_w), ptr(state), ptr(cu_q), ptr(kv_lens), ptr(slot_ids),
-                               kv_lens.numel(), rows, H, G, D, Dv, float(eps), ptr(out), out.stride(0), stream()),
+                               kv_lens.numel(), rows, H, G, D, Dv, float(eps), ptr(scratch), ptr(out), out.stride(0),
+                               stream()),
           "mi_channel_delta")
     return out
 
