@@ -74,9 +74,9 @@ __device__ __forceinline__ void load8<float>(const float* p, int n_valid, bool v
 // ---------------------------------------------------------------------------------------------------------------
 // exact kernel: 64 x 64 tile, 256 threads, 4 x 4 outputs per thread, k ascending
 // ---------------------------------------------------------------------------------------------------------------
-template <typename TW, bool DUAL>
+template <typename TW, bool DUAL, int RT>  // RT rows per thread: a 64 x 64 tile (4) or 16 x 64 (1: few features, many rows)
 __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
-  constexpr int BM = 64, BN = 64, BK = 32, PAD = 4;
+  constexpr int BM = 16 * RT, BN = 64, BK = 32, PAD = 4;
   __shared__ float As[BK][BM + PAD];
   __shared__ float Bs[DUAL ? 2 : 1][BK][BN + PAD];
   const int tid = threadIdx.x;
@@ -94,24 +94,24 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
   const int n0 = blockIdx.x * BN;
   const int lr = tid >> 2, lk = (tid & 3) * 8;  // this thread stages 8 consecutive k of one row
   int64_t xrow = -1;
-  if (m0 + lr < m_hi) xrow = a.x_rows ? a.x_rows[m0 + lr] : m0 + lr;
+  if (lr < BM && m0 + lr < m_hi) xrow = a.x_rows ? a.x_rows[m0 + lr] : m0 + lr;
   const int wrow = n0 + lr < a.N ? n0 + lr : -1;
-  float acc[DUAL ? 2 : 1][4][4] = {};
+  float acc[DUAL ? 2 : 1][RT][4] = {};
   const int ty = tid >> 4, tx = tid & 15;
   for (int k0 = 0; k0 < a.K; k0 += BK) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int k = k0 + lk + i;
-      As[lk + i][lr] = (xrow >= 0 && k < a.K) ? a.x[xrow * a.ldx + k] : 0.f;
+      if (lr < BM) As[lk + i][lr] = (xrow >= 0 && k < a.K) ? a.x[xrow * a.ldx + k] : 0.f;
       Bs[0][lk + i][lr] = (wrow >= 0 && k < a.K) ? w_load<TW>(w + (int64_t)wrow * a.K + k) : 0.f;
       if (DUAL) Bs[1][lk + i][lr] = (wrow >= 0 && k < a.K) ? w_load<TW>(w2 + (int64_t)wrow * a.K + k) : 0.f;
     }
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < BK; ++k) {
-      float av[4], bv[DUAL ? 2 : 1][4];
+      float av[RT], bv[DUAL ? 2 : 1][4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) av[i] = As[k][ty * 4 + i];
+      for (int i = 0; i < RT; ++i) av[i] = As[k][ty * RT + i];
 #pragma unroll
       for (int d = 0; d < (DUAL ? 2 : 1); ++d)
 #pragma unroll
@@ -119,15 +119,15 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
 #pragma unroll
       for (int d = 0; d < (DUAL ? 2 : 1); ++d)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < RT; ++i)
 #pragma unroll
           for (int j = 0; j < 4; ++j) acc[d][i][j] = fmaf(av[i], bv[d][j], acc[d][i][j]);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = m0 + ty * 4 + i;
+  for (int i = 0; i < RT; ++i) {
+    const int m = m0 + ty * RT + i;
     if (m >= m_hi) continue;
     const int64_t yrow = a.y_rows ? a.y_rows[m] : m;
 #pragma unroll
@@ -485,7 +485,11 @@ static int launch_any(const GemmAnyArgs& a, int groups, int rows_per_group_max, 
       return check_launch();
     }
   }
-  hipLaunchKernelGGL((gemm_any_fma_kernel<TW, DUAL>), grid, dim3(256), 0, st, a);
+  if (a.N <= 64 && rows_per_group_max >= 1024) {  // a router over a prompt: one column of tiles - short tiles, more of them
+    hipLaunchKernelGGL((gemm_any_fma_kernel<TW, DUAL, 1>), dim3(1, (rows_per_group_max + 15) / 16, groups), dim3(256), 0, st, a);
+    return check_launch();
+  }
+  hipLaunchKernelGGL((gemm_any_fma_kernel<TW, DUAL, 4>), grid, dim3(256), 0, st, a);
   return check_launch();
 }
 

@@ -101,7 +101,7 @@ def test_router_many_outputs(n, experts, top, count, keep):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 70, 33), (3, 5, 129), (8, 64, 64), (9, 65, 31), (200, 130, 200), (64, 64, 32),
-                                   (600, 200, 100), (513, 128, 64), (40, 300, 264), (4, 50, 1100), (70, 33, 1100)])
+                                   (600, 200, 100), (513, 128, 64), (40, 300, 264), (4, 50, 1100), (70, 33, 1100), (1100, 40, 70)])
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 def test_gemm_any_shapes(M, N, K, wdtype):
     from nanovllm import ops
