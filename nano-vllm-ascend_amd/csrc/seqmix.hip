@@ -377,6 +377,153 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
   }
 }
 
+// The matrix-core form for prompt portions over a bf16 cache (D a multiple of 32, Dv of 16): a wave takes 16 consecutive
+// step rows of one head.  S^T = K Q^T on v_mfma_f32_16x16x32_bf16 with the KEYS on the row axis (the A operand is a key's
+// cache row as stored: 16-byte loads), 32 keys per round; O^T += V^T P^T with the contraction slots ordered as the score
+// registers are (slot 8 g + e of lane group g = key 4 g + e of the first 16-key tile for e < 4, of the second for
+// e >= 4), so the softmax weights go from the accumulators into the B operand without leaving their lane; the V^T
+// operand gathers its eight keys' elements.  Scores and weights stay fp32 quantities: q and p enter the MFMAs as
+// bf16 hi + lo pairs (two MFMAs each, products exact, fp32 accumulation: 16 mantissa bits of q and p against the 8 of a
+// plain bf16 operand), scale, distance bias, mask, running maximum and sum are fp32 VALU work on the accumulators.
+template <int DKM, int DVM>
+__global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __restrict__ q, int64_t ldq,
+                                                                 const uint16_t* __restrict__ k_cache,
+                                                                 const uint16_t* __restrict__ v_cache,
+                                                                 const int32_t* __restrict__ block_tables, int table_cols,
+                                                                 const int32_t* __restrict__ cu_q,
+                                                                 const int32_t* __restrict__ kv_lens, int n_seqs,
+                                                                 int n_rows, int H, int G, int D, int Dv, int block_size,
+                                                                 int window, float scale, const float* __restrict__ gate,
+                                                                 int64_t ldg, float* __restrict__ out, int64_t ldo) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wid = blockIdx.x * 4 + wave;
+  const int n_groups = (n_rows + 15) / 16;
+  if (wid >= n_groups * H) return;
+  const int rg = wid / H, h = wid % H;
+  const int g = h / (H / G);
+  const float slope = exp2f(-8.f * (float)(h + 1) / (float)H);
+  const int qi = lane & 15, kg = lane >> 4;
+  const int dk = D / 32, dvt = Dv / 16;
+  const bool q_vec = (ldq % 4 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15u) == 0) && (D % 4 == 0);
+  const int group_end = min(rg * 16 + 16, n_rows);
+  for (int first = rg * 16; first < group_end;) {
+    const int s = seq_of_row(cu_q, n_seqs, first);
+    const int end = min(cu_q[s + 1], group_end), nr = end - first;
+    const int pos0 = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (first - cu_q[s]);
+    const int32_t* table = block_tables + (int64_t)s * table_cols;
+    bf16x8 qh[DKM], ql[DKM];
+#pragma unroll
+    for (int ks = 0; ks < DKM; ++ks) {
+      float xv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (ks < dk && qi < nr) {
+        const float* qp = q + (int64_t)(first + qi) * ldq + h * D + ks * 32 + kg * 8;
+        if (q_vec) {
+          const float4 a = *reinterpret_cast<const float4*>(qp), b = *reinterpret_cast<const float4*>(qp + 4);
+          xv[0] = a.x, xv[1] = a.y, xv[2] = a.z, xv[3] = a.w, xv[4] = b.x, xv[5] = b.y, xv[6] = b.z, xv[7] = b.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) xv[e] = qp[e];
+        }
+      }
+      float lo[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) lo[e] = xv[e] - rbf(xv[e]);
+      qh[ks] = as_frag(u32x4{pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])});
+      ql[ks] = as_frag(u32x4{pack_bf(lo[0], lo[1]), pack_bf(lo[2], lo[3]), pack_bf(lo[4], lo[5]), pack_bf(lo[6], lo[7])});
+    }
+    const int lo_key = max(0, pos0 - window + 1), hi_key = pos0 + nr - 1;
+    const int my_pos = pos0 + qi;
+    float m = -INFINITY, l = 0.f;
+    f32x4 oacc[DVM];
+#pragma unroll
+    for (int dt = 0; dt < DVM; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j0 = lo_key; j0 <= hi_key; j0 += 32) {
+      f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int key = j0 + t * 16 + qi;  // (this lane's row of the K operand)
+        const bool ok = key <= hi_key;
+        const uint16_t* kr = k_cache;
+        if (ok) kr += (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
+#pragma unroll
+        for (int ks = 0; ks < DKM; ++ks) {
+          if (ks < dk) {
+            u32x4 kv = {0u, 0u, 0u, 0u};
+            if (ok) kv = *reinterpret_cast<const u32x4*>(kr + ks * 32);
+            const bf16x8 kf = as_frag(kv);
+            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qh[ks], sacc[t], 0, 0, 0);
+            sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[ks], sacc[t], 0, 0, 0);
+          }
+        }
+      }
+      float sc[8];
+      bool vis[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
+        vis[e] = qi < nr && key <= my_pos && key > my_pos - window;
+        sc[e] = vis[e] ? sacc[e >> 2][e & 3] * scale - slope * (float)(my_pos - key) : -INFINITY;
+        mx = fmaxf(mx, sc[e]);
+      }
+      mx = xor_max<32>(xor_max<16>(mx));
+      const float m_new = fmaxf(m, mx);
+      const float corr = m == -INFINITY ? 0.f : expf(m - m_new);
+      float pv[8], psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = vis[e] ? expf(sc[e] - m_new) : 0.f;
+        psum += pv[e];
+      }
+      psum = xor_sum<32>(xor_sum<16>(psum));
+      l = l * corr + psum;
+      m = m_new;
+      float plo[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) plo[e] = pv[e] - rbf(pv[e]);
+      const bf16x8 ph = as_frag(u32x4{pack_bf(pv[0], pv[1]), pack_bf(pv[2], pv[3]), pack_bf(pv[4], pv[5]), pack_bf(pv[6], pv[7])});
+      const bf16x8 pl = as_frag(u32x4{pack_bf(plo[0], plo[1]), pack_bf(plo[2], plo[3]), pack_bf(plo[4], plo[5]), pack_bf(plo[6], plo[7])});
+      const uint16_t* vrow[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
+        vrow[e] = key <= hi_key
+                      ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * Dv + qi
+                      : nullptr;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DVM; ++dt) {
+        if (dt < dvt) {
+          uint32_t ve[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ve[e] = vrow[e] ? (uint32_t)vrow[e][dt * 16] : 0u;
+          const bf16x8 vf = as_frag(u32x4{ve[0] | (ve[1] << 16), ve[2] | (ve[3] << 16), ve[4] | (ve[5] << 16), ve[6] | (ve[7] << 16)});
+          oacc[dt] *= corr;
+          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, oacc[dt], 0, 0, 0);
+          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, oacc[dt], 0, 0, 0);
+        }
+      }
+    }
+    if (qi < nr) {  // the lane holds channels 16 dt + 4 kg + r of its query's output
+      const float inv = 1.f / l;
+      const int64_t row = first + qi;
+#pragma unroll
+      for (int dt = 0; dt < DVM; ++dt) {
+        if (dt < dvt) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int d = dt * 16 + kg * 4 + r;
+            float o = oacc[dt][r] * inv;
+            if (gate) o *= sigmoid_f(gate[row * ldg + h * Dv + d]);
+            out[row * ldo + h * Dv + d] = o;
+          }
+        }
+      }
+    }
+    first = end;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // short causal convolution with a carried tail
 // ---------------------------------------------------------------------------------------------------------------
@@ -765,6 +912,19 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
   const TC* k = static_cast<const TC*>(kc);
   const TC* v = static_cast<const TC*>(vc);
   constexpr int VEC = 16 / sizeof(TC);
+  if constexpr (sizeof(TC) == 2) {
+    // prompt portions over a bf16 cache: the matrix-core form
+    if (rows > n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256) {
+      const dim3 grid_m((((rows + 15) / 16) * H + 3) / 4);
+      if (D <= 128 && Dv <= 128)
+        hipLaunchKernelGGL((swa_attention_mfma_kernel<4, 8>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,
+                           n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo);
+      else
+        hipLaunchKernelGGL((swa_attention_mfma_kernel<8, 16>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,
+                           n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo);
+      return check_launch();
+    }
+  }
   if (D % VEC == 0 && Dv % VEC == 0 && Dv / VEC <= 64) {
     int lpr_log2 = 0;
     while ((1 << lpr_log2) * VEC < Dv) ++lpr_log2;

@@ -85,6 +85,37 @@ def test_router_choices_and_weights():
     assert (wts.sum(-1) < 0.999).any()       # not renormalised
 
 
+@pytest.mark.parametrize("H,G,D,Dv,window,T,start", [(4, 2, 64, 48, 70, 200, 0), (2, 2, 128, 128, 33, 90, 57), (8, 1, 32, 16, 300, 150, 0),
+                                                     (2, 1, 256, 160, 40, 70, 5)])
+def test_window_attention_on_the_matrix_cores(H, G, D, Dv, window, T, start):
+    """The MFMA form of the window attention (prompt portions over a bf16 cache) at the operator level: q and the softmax
+    weights enter the matrix cores as bf16 hi + lo pairs, so the result stays at fp32 quality (1e-4 of the output's size;
+    a plain bf16 q or p would show as 4e-3).  Scattered pages; a portion that continues `start` cached tokens."""
+    from nanovllm import ops
+
+    g = torch.Generator().manual_seed(D + T)
+    bs, n = 16, start + T
+    k = torch.randn(n, G, D, generator=g).bfloat16()
+    v = torch.randn(n, G, Dv, generator=g).bfloat16()
+    q = torch.randn(n, H, D, generator=g)
+    n_blocks = -(-n // bs)
+    table = torch.randperm(n_blocks + 3, generator=g)[:n_blocks].to(torch.int32)
+    kc = torch.zeros(n_blocks + 3, G, bs, D, dtype=torch.bfloat16)
+    vc = torch.zeros(n_blocks + 3, G, bs, Dv, dtype=torch.bfloat16)
+    for p in range(n):
+        kc[table[p // bs], :, p % bs] = k[p]
+        vc[table[p // bs], :, p % bs] = v[p]
+    want = G_windowed(q, k, v, 0.17, window)[start:]
+    got = ops.swa_attention(q[start:].reshape(T, H * D).contiguous().cuda(), kc.cuda(), vc.cuda(), table.view(1, -1).cuda(),
+                            torch.tensor([0, T], dtype=torch.int32).cuda(), torch.tensor([n], dtype=torch.int32).cuda(),
+                            H, G, D, Dv, bs, window, 0.17).cpu().double().view(T, H, Dv)
+    assert (got - want).abs().max() <= 1e-4 * want.abs().max(), float((got - want).abs().max() / want.abs().max())
+
+
+def G_windowed(q, k, v, scale, window):
+    return G.windowed_attention(q.double(), k.double(), v.double(), scale, window)
+
+
 @pytest.mark.parametrize("n,experts,top,count,keep", [(130, 128, 6, 10, 3), (130, 126, 9, 65, 7), (512, 500, 8, 8, 2)])
 def test_router_many_outputs(n, experts, top, count, keep):
     """More router outputs than lanes (several per lane), more groups than lanes."""
