@@ -55,6 +55,8 @@ def run_worker(model, **kwargs) -> None:
 
 
 class LLMEngine:
+    _chunked_rows = False  # (engines assembled without __init__ - the host tests' scripted engines - step the classic way)
+
     def __init__(self, model, **kwargs):
         config = _make_config(model, kwargs)
         self.config = config
@@ -77,6 +79,8 @@ class LLMEngine:
         # running is scheduled and queued on the device(s) before the running one's tokens reach the host; the TP
         # workers queue the same step when its message arrives (ModelRunner.loop)
         self.lookahead = config.decode_lookahead and os.environ.get("MI355_LOOKAHEAD", "1") != "0"
+        # hybrid models with Config.chunked_prefill: every step is a list of row runs (Scheduler.schedule_rows)
+        self._chunked_rows = bool(config.hybrid_state and config.chunked_prefill)
         self._inflight = None  # (handle, sequences, rows dropped after launch) of a queued decode step
         # ... and the same between consecutive PREFILL steps (one GPU): while a long prefill step runs, the next one is
         # admitted (Scheduler.lookahead_prefill: only when that is the decision schedule() would take afterwards) and
@@ -236,7 +240,7 @@ class LLMEngine:
         if self._inflight_prefill is not None:
             queued, self._inflight_prefill = self._inflight_prefill, None
             return self._step_prefill(*queued)
-        if self.config.hybrid_state and self.config.chunked_prefill:
+        if self._chunked_rows:
             return self._step_rows()
         seqs, is_prefill = self.scheduler.schedule()
         if self.lookahead and not is_prefill and seqs and self.model_runner.can_launch_decode(len(seqs)):
