@@ -5,14 +5,16 @@
 // These serve the model families whose residual stream, norms and recurrences are kept in 32-bit floats and whose
 // widths are not the fragment-native kernels' (csrc/gemm_skinny*.hpp, gemm_tile.hip): four kernels,
 //
-//   gemm_any_mfma_kernel   bf16 weights: 64 x 64 output tile per 4-wave workgroup, x rounded to bf16 on its way into
-//                          LDS, v_mfma_f32_16x16x32_bf16, edges zero-filled by guarded loads
+//   gemm_any_mfma_kernel   bf16 weights: a 64 x 64 (from 512 rows: 128 x 128, with SwiGLU 128 x 64) output tile per 4-wave
+//                          workgroup, x rounded to bf16 on its way into LDS, v_mfma_f32_16x16x32_bf16, the next K
+//                          step's operands fetched while the current one is multiplied, edges zero-filled
 //   gemm_any_skinny_kernel bf16 weights, up to 64 rows per tile (decode batches, a decode step's experts): 16 features per
 //                          workgroup, the waves split K, fragments straight from memory
 //   gemm_any_fma_kernel    true 32-bit: fp32 (or bf16, widened exactly) weights, x NOT rounded, plain FMA chains in k
 //                          order - the float32 serving mode, and the routers of sparse feed-forwards in either mode
-//   gemm_any_rows_kernel   M <= 8 rows (decode): one wave per output feature streams its weight row once, lanes
-//                          split K in 16-byte pieces, butterfly reduction; both dtypes, x not rounded
+//   gemm_any_rows_kernel   M <= 8 rows, and the exact mode up to 64: one wave per (output feature, batch of rows)
+//                          streams its weight row once, lanes split K in 16-byte pieces, butterfly reduction; both
+//                          dtypes, x not rounded
 //
 // A row of the result is a function of its own x row and the weights only: the summation order over k does not depend
 // on M, on the row's place in the batch or on the tile it falls into (each kernel has ONE fixed order), so the same

@@ -10,7 +10,8 @@
 //                               s_ij = scale q_i.k_j - slope_h (i - j), keys 0 <= i - j < window, separate key and value
 //                               head sizes, grouped heads, optional sigmoid output gate; prompt portions and single
 //                               decoded tokens in one launch (a row's keys are addressed through its sequence's block
-//                               table and total length)
+//                               table and total length); three kernels: matrix cores for prompt portions over a bf16
+//                               cache, 16-byte-load VALU form (decode: four waves per row and head), element-wise form
 //   mi_causal_conv_silu         short causal depthwise convolution over time + SiLU, carried across steps by a
 //   mi_causal_conv_state        per-sequence state slot holding the last taps - 1 inputs
 //   mi_channel_delta            gated delta rule with one decay per head AND key channel:
@@ -22,7 +23,8 @@
 //   mi_moe_combine_f32          out[t] = sum_k w[t][k] * (identity expert ? h[t] : y[t * top_k + k])
 //
 // Everything here is computed in fp32 (expf / logf / sqrtf of the device library, no fast-math), for both serving
-// dtypes: the bf16 mode differs only in the dtype of the WEIGHTS and of the K/V cache.
+// dtypes: the bf16 mode differs only in the dtype of the WEIGHTS and of the K/V cache (and in the matrix-core attention
+// of prompt portions, whose two products take q and the softmax weights as bf16 hi + lo pairs: fp32 quantities to 2^-17).
 // A step's rows are described by cu_q [n_seqs + 1] (row range of each sequence) and kv_lens [n_seqs] (the sequence's
 // length INCLUDING this step's rows): row r of sequence s sits at position kv_lens[s] - (cu_q[s+1] - cu_q[s]) + r.
 #include "mi_common.hpp"
