@@ -387,7 +387,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
 // operand gathers its eight keys' elements.  Scores and weights stay fp32 quantities: q and p enter the MFMAs as
 // bf16 hi + lo pairs (two MFMAs each, products exact, fp32 accumulation: 16 mantissa bits of q and p against the 8 of a
 // plain bf16 operand), scale, distance bias, mask, running maximum and sum are fp32 VALU work on the accumulators.
-template <int DKM, int DVM>
+template <int DKM, int DVM, bool PAIR>
 __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __restrict__ q, int64_t ldq,
                                                                  const uint16_t* __restrict__ k_cache,
                                                                  const uint16_t* __restrict__ v_cache,
@@ -485,28 +485,55 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
       for (int e = 0; e < 8; ++e) plo[e] = pv[e] - rbf(pv[e]);
       const bf16x8 ph = as_frag(u32x4{pack_bf(pv[0], pv[1]), pack_bf(pv[2], pv[3]), pack_bf(pv[4], pv[5]), pack_bf(pv[6], pv[7])});
       const bf16x8 pl = as_frag(u32x4{pack_bf(plo[0], plo[1]), pack_bf(plo[2], plo[3]), pack_bf(plo[4], plo[5]), pack_bf(plo[6], plo[7])});
+      // V^T operand: the lane's eight keys (its contraction slots) at ONE channel per 16-channel tile - or, when Dv is a
+      // multiple of 32 (PAIR), at TWO neighbouring channels per 32-channel pair of tiles with one 4-byte load: the low
+      // halves feed the tile of the pair's even channels, the high halves the tile of its odd channels
       const uint16_t* vrow[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
         vrow[e] = key <= hi_key
-                      ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * Dv + qi
+                      ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * Dv +
+                            (PAIR ? 2 * qi : qi)
                       : nullptr;
       }
+      if constexpr (PAIR) {
 #pragma unroll
-      for (int dt = 0; dt < DVM; ++dt) {
-        if (dt < dvt) {
-          uint32_t ve[8];
+        for (int dp = 0; dp < DVM / 2; ++dp) {
+          if (2 * dp < dvt) {
+            uint32_t w[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) ve[e] = vrow[e] ? (uint32_t)vrow[e][dt * 16] : 0u;
-          const bf16x8 vf = as_frag(u32x4{ve[0] | (ve[1] << 16), ve[2] | (ve[3] << 16), ve[4] | (ve[5] << 16), ve[6] | (ve[7] << 16)});
-          oacc[dt] *= corr;
-          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, oacc[dt], 0, 0, 0);
-          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, oacc[dt], 0, 0, 0);
+            for (int e = 0; e < 8; ++e) w[e] = vrow[e] ? *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32) : 0u;
+            const bf16x8 v_even = as_frag(u32x4{(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16),
+                                                (w[4] & 0xffffu) | (w[5] << 16), (w[6] & 0xffffu) | (w[7] << 16)});
+            const bf16x8 v_odd = as_frag(u32x4{(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u),
+                                               (w[4] >> 16) | (w[5] & 0xffff0000u), (w[6] >> 16) | (w[7] & 0xffff0000u)});
+            oacc[2 * dp] *= corr;
+            oacc[2 * dp + 1] *= corr;
+            oacc[2 * dp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_even, ph, oacc[2 * dp], 0, 0, 0);
+            oacc[2 * dp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_even, pl, oacc[2 * dp], 0, 0, 0);
+            oacc[2 * dp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_odd, ph, oacc[2 * dp + 1], 0, 0, 0);
+            oacc[2 * dp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_odd, pl, oacc[2 * dp + 1], 0, 0, 0);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int dt = 0; dt < DVM; ++dt) {
+          if (dt < dvt) {
+            uint32_t ve[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ve[e] = vrow[e] ? (uint32_t)vrow[e][dt * 16] : 0u;
+            const bf16x8 vf = as_frag(u32x4{ve[0] | (ve[1] << 16), ve[2] | (ve[3] << 16), ve[4] | (ve[5] << 16), ve[6] | (ve[7] << 16)});
+            oacc[dt] *= corr;
+            oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, oacc[dt], 0, 0, 0);
+            oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, oacc[dt], 0, 0, 0);
+          }
         }
       }
     }
-    if (qi < nr) {  // the lane holds channels 16 dt + 4 kg + r of its query's output
+    if (qi < nr) {
+      // the lane holds channels 16 dt + 4 kg + r of its query's output (PAIR: tile 2 dp + b holds the channels
+      // 32 dp + 2 (4 kg + r) + b, i.e. the lane has the eight consecutive channels 32 dp + 8 kg .. + 7)
       const float inv = 1.f / l;
       const int64_t row = first + qi;
 #pragma unroll
@@ -514,7 +541,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
         if (dt < dvt) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int d = dt * 16 + kg * 4 + r;
+            const int d = PAIR ? (dt >> 1) * 32 + 2 * (kg * 4 + r) + (dt & 1) : dt * 16 + kg * 4 + r;
             float o = oacc[dt][r] * inv;
             if (gate) o *= sigmoid_f(gate[row * ldg + h * Dv + d]);
             out[row * ldo + h * Dv + d] = o;
@@ -918,12 +945,15 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
     // prompt portions over a bf16 cache: the matrix-core form
     if (rows > n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256) {
       const dim3 grid_m((((rows + 15) / 16) * H + 3) / 4);
-      if (D <= 128 && Dv <= 128)
-        hipLaunchKernelGGL((swa_attention_mfma_kernel<4, 8>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,
-                           n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo);
-      else
-        hipLaunchKernelGGL((swa_attention_mfma_kernel<8, 16>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,
-                           n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo);
+#define MI_SWA_MFMA(DKM, DVM, PAIR)                                                                                    \
+  hipLaunchKernelGGL((swa_attention_mfma_kernel<DKM, DVM, PAIR>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, \
+                     kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo)
+      const bool small = D <= 128 && Dv <= 128, pair = Dv % 32 == 0;
+      if (small && pair) MI_SWA_MFMA(4, 8, true);
+      else if (small) MI_SWA_MFMA(4, 8, false);
+      else if (pair) MI_SWA_MFMA(8, 16, true);
+      else MI_SWA_MFMA(8, 16, false);
+#undef MI_SWA_MFMA
       return check_launch();
     }
   }
