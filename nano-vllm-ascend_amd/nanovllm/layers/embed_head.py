@@ -94,10 +94,11 @@ class ParallelLMHead(VocabParallelEmbedding):
             parallel.STATS["rccl_gather"] += 1
             dist.gather(logits, parts, 0)
             return torch.cat(parts, -1) if self.tp_rank == 0 else None
-        # gloo has no device-side gather: place the shard in a zero buffer and sum (tests only)
+        # gloo has no device-side gather: place the shard in a zero buffer and sum (tests only) - on the host, where gloo's
+        # tensors belong (parallel.group_all_reduce)
         full = torch.zeros((logits.shape[0], self.num_embeddings), dtype=logits.dtype, device=logits.device)
         full[:, self.vocab_start_idx:self.vocab_end_idx] = logits
-        dist.all_reduce(full)
+        parallel.group_all_reduce(full)
         return full if self.tp_rank == 0 else None
 
     def forward(self, x: torch.Tensor):

@@ -76,6 +76,20 @@ def get_xgmi_comm():
     return _xgmi
 
 
+def group_all_reduce(t, op=None):
+    """dist.all_reduce in place on whatever backend the group has.  gloo gets CPU tensors only: a device tensor is copied
+    to host memory with a synchronous copy, reduced there and copied back - gloo's collectives on device tensors have
+    hung when several ranks shared one GPU (the functional tensor-parallel runs of a one-GPU box)."""
+    kw = {} if op is None else {"op": op}
+    if t.is_cuda and dist.get_backend() == "gloo":
+        host = t.cpu()
+        dist.all_reduce(host, **kw)
+        t.copy_(host)
+    else:
+        dist.all_reduce(t, **kw)
+    return t
+
+
 def all_reduce_sum(t):
     """C1/C2 of SURVEY.md §2.2: SUM over the TP ranks, in place.  Decode-sized bf16 vectors take
     the one-shot xGMI kernel (mi_allreduce_sum_bf16, hipGraph-capturable, one launch); everything
@@ -84,5 +98,5 @@ def all_reduce_sum(t):
         if _xgmi is not None and _xgmi.fits(t):
             return _xgmi.all_reduce(t)
         STATS["rccl_all_reduce"] += 1
-        dist.all_reduce(t)
+        group_all_reduce(t)
     return t
