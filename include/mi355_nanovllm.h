@@ -712,6 +712,74 @@ int mi_route_grouped(const float* logits, int64_t ld, const float* correction, i
 int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, const int32_t* ids, const float* weights,
                        int n_tokens, int top_k, int n_experts, int width, float* out, int64_t ldo, mi_stream stream);
 
+/* Epilogue activations of mi_gemm_any_act / mi_gemm_any_grouped_act. */
+#define MI_ACT_NONE      0
+#define MI_ACT_SILU      1
+#define MI_ACT_GELU_TANH 2  /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */
+#define MI_ACT_GELU_ERF  3  /* 0.5 z (1 + erf(z / sqrt 2)) */
+#define MI_ACT_SIGMOID   4
+/* mi_gemm_any with an epilogue: v = x w^T + bias (bias may be NULL); w2 != NULL: y = alpha * act(v) * (x w2^T + bias2),
+ * else y = alpha * act(v). */
+int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const void* w2, int w_dtype, const float* bias,
+                    const float* bias2, int act, float* y, int64_t ldy, int M, int N, int K, float alpha, int exact,
+                    mi_stream stream);
+/* mi_gemm_any_grouped with the activation named: y = act(x w^T) (* (x w2^T) with w2). */
+int mi_gemm_any_grouped_act(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2, int w_dtype,
+                            int act, const int32_t* group_offsets, int n_groups, int rows_per_group_max, float* y,
+                            int64_t ldy, const int32_t* y_rows, int N, int K, int exact, mi_stream stream);
+/* n_batch products over the same M rows: batch b: y + b*y_batch [M][N] (ldy) = (x + b*x_batch) [M][K] (ldx) . w[b]^T
+ * (w = [n_batch][N][K]) - a projection per head of head-major rows.  gate != NULL: times
+ * sigmoid((gate + b*gate_batch)[row][n]) (ldgate). */
+int mi_gemm_any_batched(const float* x, int64_t ldx, int64_t x_batch, const void* w, int w_dtype, float* y, int64_t ldy,
+                        int64_t y_batch, const float* gate, int64_t ldgate, int64_t gate_batch, int n_batch, int M, int N,
+                        int K, int exact, mi_stream stream);
+/* Distance bias of mi_paged_attention_f32, taken off the scaled score; dist = i - j >= 0: */
+#define MI_BIAS_SLOPE 0  /* p1[h] * dist; p1 == NULL: 2^(-8 (h+1) / H) * dist */
+#define MI_BIAS_LOG   1  /* p1[h] * ln(1 + p2[h] * dist) */
+#define MI_BIAS_NONE  2
+/* mi_swa_attention with the bias named and the value rows ldv elements apart: v_cache may be k_cache itself with
+ * ldv = D when a token's value is the first Dv channels of its key row (latent attention: G = 1).  window >= the longest
+ * sequence: plain causal attention. */
+int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
+                           int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
+                           const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv, int block_size,
+                           int window, float scale, int bias_kind, const float* bias_p1, const float* bias_p2,
+                           const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream);
+/* res += mult * y (y may be NULL); w != NULL: out = res / sqrt(mean(res^2) + eps) * (w + shift) per row. */
+int mi_add_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* w, float shift,
+                       float eps, float* out, int64_t ldo, int rows, int width, mi_stream stream);
+/* stack = slots [rows][width] of the layers' results, slot_stride floats apart.  Slot n-1 += mult * y (y may be NULL);
+ * slot n = sum_{j<n} coef[j] * slot j; norm_w != NULL: h = slot n / rms * (norm_w + shift). */
+int mi_depth_mix_f32(float* stack, int64_t slot_stride, int n, const float* coef, const float* y, int64_t ldy, float mult,
+                     const float* norm_w, float shift, float eps, float* h, int64_t ldh, int rows, int width,
+                     mi_stream stream);
+/* Minimal gated recurrence per channel: z = sigmoid(proj[z_off + c]), u = proj[x_off + c], cand = u + 1/2 (u >= 0) or
+ * sigmoid(u); S <- (1 - z) S + z cand; out = S * silu(proj[g_off + c]).  state [slots][width] fp32.  Steps with more than
+ * 64 rows of a sequence run as parallel segments (workspace: mi_mingru_scan_workspace_elems floats). */
+int64_t mi_mingru_scan_workspace_elems(int rows, int n_seqs, int width);
+int mi_mingru_scan(const float* proj, int64_t ld, int z_off, int x_off, int g_off, float* state, const int32_t* cu_q,
+                   const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows, int max_rows_per_seq, int width,
+                   float* workspace, float* out, int64_t ldo, mi_stream stream);
+/* q (H*D at q_off) *= 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1) in place (temp_every < 1: unchanged); k, v
+ * rows to caches [blocks][G][block_size][D | Dv]. */
+int mi_kv_store_temp(float* proj, int64_t ld, int q_off, int k_off, int v_off, float temp_coef, int temp_every,
+                     const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, void* k_cache, void* v_cache, int cache_dtype,
+                     const int32_t* slots, int rows, int H, int G, int D, int Dv, int block_size, mi_stream stream);
+/* Latent attention, per row: cache row [slot] = [rms(c) * norm_w | rot(r)] (c: C entries at c_off, r: the R behind
+ * them); qx[row][h][C .. C + R) = rot(q_h[D .. D + R)) for every head (q heads of D + R entries at q_off).  rot turns
+ * the first rot_dims entries: pairs (i, i + rot_dims/2), angle pos * rot_base^(-2 i / rot_dims). */
+int mi_latent_prepare(const float* proj, int64_t ld, int q_off, int c_off, int H, int D, int R, int C, int rot_dims,
+                      float rot_base, const float* norm_w, float eps, const int32_t* cu_q, const int32_t* kv_lens,
+                      int n_seqs, void* cache, int cache_dtype, const int32_t* slots, float* qx, int64_t ldqx, int rows,
+                      mi_stream stream);
+/* ids = the top_k largest logits (descending; equal: lower index), weights = softmax over those.  n_outputs <= 512. */
+int mi_route_topk(const float* logits, int64_t ld, int n_tokens, int n_outputs, int top_k, int32_t* ids, float* weights,
+                  mi_stream stream);
+/* out[t] = sum_k weights[t][k] * y[t * top_k + k] + sigmoid(shared_gate[t]) * shared[t] (shared may be NULL). */
+int mi_moe_combine_shared(const float* y, const int32_t* ids, const float* weights, int n_tokens, int top_k, int width,
+                          const float* shared, int64_t ld_shared, const float* shared_gate, int64_t ld_gate, float* out,
+                          int64_t ldo, mi_stream stream);
+
 /* ---- host-side hashing (reference: engine/block_manager.py:38-44) --------- */
 /* xxh64 of `len` bytes with seed 0, optionally prefixed by the 8 little-endian
  * bytes of `prefix` (has_prefix != 0) — the chained block hash of

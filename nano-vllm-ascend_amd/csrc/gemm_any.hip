@@ -36,6 +36,16 @@ struct GemmAnyArgs {
   const int32_t* group_offsets;  // nullptr: one group of M rows; else rows of group g = [off[g], off[g + 1])
   const int32_t* x_rows;         // nullptr or the x row of each (sorted) row
   const int32_t* y_rows;         // nullptr or the y row of each (sorted) row
+  // epilogue: v = acc + bias[n]; with w2: v = act(v) * (acc2 + bias2[n]), else v = act(v); v *= alpha;
+  // gate: v *= sigmoid(gate[y row][n])
+  const float* bias;
+  const float* bias2;
+  int act;  // MI_ACT_*
+  const float* gate;
+  int64_t ldgate;
+  // batched form (group_offsets == nullptr, gridDim.z > 1): batch b multiplies the M rows at x + b * x_batch with
+  // w[b] into y + b * y_batch (a per-head projection of head-major rows: the batch stride is a head's width)
+  int64_t x_batch, y_batch, gate_batch;
 };
 
 template <typename TW>
@@ -47,6 +57,46 @@ __device__ __forceinline__ float w_load<uint16_t>(const uint16_t* p) { return bf
 
 __device__ __forceinline__ bool dev_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float act_f(int act, float z) {
+  switch (act) {
+    case MI_ACT_SILU: return silu_f(z);
+    case MI_ACT_GELU_TANH: return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    case MI_ACT_GELU_ERF: return 0.5f * z * (1.f + erff(z * 0.7071067811865476f));
+    case MI_ACT_SIGMOID: return 1.f / (1.f + expf(-z));
+    default: return z;
+  }
+}
+// what every kernel does to an accumulator (pair) before it stores it
+template <bool DUAL>
+__device__ __forceinline__ float finish(const GemmAnyArgs& a, int64_t yrow, int n, float v, float v2) {
+  if (a.bias) v += a.bias[n];
+  if (DUAL) {
+    if (a.bias2) v2 += a.bias2[n];
+    v = act_f(a.act, v) * v2;
+  } else {
+    v = act_f(a.act, v);
+  }
+  v *= a.alpha;
+  if (a.gate) v *= 1.f / (1.f + expf(-a.gate[yrow * a.ldgate + n]));
+  return v;
+}
+// the operands of this workgroup's group (grouped form) or batch (batched form)
+template <typename TW, bool DUAL>
+__device__ __forceinline__ void select_group(GemmAnyArgs& a, const TW*& w, const TW*& w2, int& m_lo, int& m_hi) {
+  m_lo = 0, m_hi = a.M;
+  w = static_cast<const TW*>(a.w);
+  w2 = static_cast<const TW*>(a.w2);
+  if (a.group_offsets) {
+    m_lo = a.group_offsets[blockIdx.z];
+    m_hi = a.group_offsets[blockIdx.z + 1];
+  } else if (blockIdx.z > 0) {
+    a.x += (int64_t)blockIdx.z * a.x_batch;
+    a.y += (int64_t)blockIdx.z * a.y_batch;
+    if (a.gate) a.gate += (int64_t)blockIdx.z * a.gate_batch;
+  }
+  w += (int64_t)blockIdx.z * a.N * a.K;
+  if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
+}
 
 // eight consecutive operands as floats: one 16-byte (bf16) / two 16-byte (fp32) loads, or element-wise at an edge
 template <typename TW>
@@ -82,15 +132,9 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
   __shared__ float As[BK][BM + PAD];
   __shared__ float Bs[DUAL ? 2 : 1][BK][BN + PAD];
   const int tid = threadIdx.x;
-  int m_lo = 0, m_hi = a.M;
-  const TW* w = static_cast<const TW*>(a.w);
-  const TW* w2 = static_cast<const TW*>(a.w2);
-  if (a.group_offsets) {
-    m_lo = a.group_offsets[blockIdx.z];
-    m_hi = a.group_offsets[blockIdx.z + 1];
-    w += (int64_t)blockIdx.z * a.N * a.K;
-    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
-  }
+  int m_lo, m_hi;
+  const TW *w, *w2;
+  select_group<TW, DUAL>(a, w, w2, m_lo, m_hi);
   const int m0 = m_lo + blockIdx.y * BM;
   if (m0 >= m_hi) return;
   const int n0 = blockIdx.x * BN;
@@ -136,9 +180,7 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(GemmAnyArgs a) {
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= a.N) continue;
-      float v = acc[0][i][j];
-      if (DUAL) v = silu_f(v) * acc[1][i][j];
-      a.y[yrow * a.ldy + n] = v * a.alpha;
+      a.y[yrow * a.ldy + n] = finish<DUAL>(a, yrow, n, acc[0][i][j], acc[DUAL ? 1 : 0][i][j]);
     }
   }
 }
@@ -156,15 +198,9 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t As[BM][LD];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[ND][BN][LD];
   const int tid = threadIdx.x;
-  int m_lo = 0, m_hi = a.M;
-  const uint16_t* w = static_cast<const uint16_t*>(a.w);
-  const uint16_t* w2 = static_cast<const uint16_t*>(a.w2);
-  if (a.group_offsets) {
-    m_lo = a.group_offsets[blockIdx.z];
-    m_hi = a.group_offsets[blockIdx.z + 1];
-    w += (int64_t)blockIdx.z * a.N * a.K;
-    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
-  }
+  int m_lo, m_hi;
+  const uint16_t *w, *w2;
+  select_group<uint16_t, DUAL>(a, w, w2, m_lo, m_hi);
   const int m0 = m_lo + blockIdx.y * BM;
   if (m0 >= m_hi) return;
   const int n0 = blockIdx.x * BN;
@@ -275,11 +311,8 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(GemmAnyArgs a) {
       const int n = n0 + wn + j * 16 + (lane >> 4) * 4;
       float v[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        v[r] = acc[0][i][j][r];
-        if (DUAL) v[r] = silu_f(v[r]) * acc[ND - 1][i][j][r];
-        v[r] *= a.alpha;
-      }
+      for (int r = 0; r < 4; ++r)
+        v[r] = n + r < a.N ? finish<DUAL>(a, yrow, n + r, acc[0][i][j][r], acc[ND - 1][i][j][r]) : 0.f;
       float* yp = a.y + yrow * a.ldy + n;
       if (n + 4 <= a.N && (a.ldy % 4 == 0) && dev_aligned16(a.y)) {
         *reinterpret_cast<float4*>(yp) = float4{v[0], v[1], v[2], v[3]};
@@ -302,15 +335,9 @@ template <bool DUAL, int MF>  // MF fragments of 16 rows
 __global__ __launch_bounds__(256) void gemm_any_skinny_kernel(GemmAnyArgs a) {
   __shared__ __attribute__((aligned(16))) float red[3][DUAL ? 2 : 1][MF][64][4];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  int m_lo = 0, m_hi = a.M;
-  const uint16_t* w = static_cast<const uint16_t*>(a.w);
-  const uint16_t* w2 = static_cast<const uint16_t*>(a.w2);
-  if (a.group_offsets) {
-    m_lo = a.group_offsets[blockIdx.z];
-    m_hi = a.group_offsets[blockIdx.z + 1];
-    w += (int64_t)blockIdx.z * a.N * a.K;
-    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
-  }
+  int m_lo, m_hi;
+  const uint16_t *w, *w2;
+  select_group<uint16_t, DUAL>(a, w, w2, m_lo, m_hi);
   const int m0 = m_lo + blockIdx.y * 16 * MF;
   if (m0 >= m_hi) return;
   const int n0 = blockIdx.x * 16;
@@ -387,9 +414,7 @@ __global__ __launch_bounds__(256) void gemm_any_skinny_kernel(GemmAnyArgs a) {
     for (int r = 0; r < 4; ++r) {
       const int n = n0 + (lane >> 4) * 4 + r;
       if (n >= a.N) continue;
-      float v = acc[0][f][r];
-      if (DUAL) v = silu_f(v) * acc[DUAL ? 1 : 0][f][r];
-      a.y[yrow * a.ldy + n] = v * a.alpha;
+      a.y[yrow * a.ldy + n] = finish<DUAL>(a, yrow, n, acc[0][f][r], acc[DUAL ? 1 : 0][f][r]);
     }
   }
 }
@@ -402,15 +427,9 @@ template <typename TW, int MT, bool DUAL>
 __global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
   const int lane = threadIdx.x & 63;
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  int m_lo = 0, m_hi = a.M;
-  const TW* w = static_cast<const TW*>(a.w);
-  const TW* w2 = static_cast<const TW*>(a.w2);
-  if (a.group_offsets) {
-    m_lo = a.group_offsets[blockIdx.z];
-    m_hi = a.group_offsets[blockIdx.z + 1];
-    w += (int64_t)blockIdx.z * a.N * a.K;
-    if (DUAL) w2 += (int64_t)blockIdx.z * a.N * a.K;
-  }
+  int m_lo, m_hi;
+  const TW *w, *w2;
+  select_group<TW, DUAL>(a, w, w2, m_lo, m_hi);
   const int m0 = m_lo + blockIdx.y * MT;
   if (n >= a.N || m0 >= m_hi) return;  // (whole waves: the reductions below see all 64 lanes)
   const bool w_vec = a.K % 8 == 0 && dev_aligned16(a.w) && (!DUAL || dev_aligned16(a.w2));
@@ -436,11 +455,11 @@ __global__ __launch_bounds__(256) void gemm_any_rows_kernel(GemmAnyArgs a) {
   }
 #pragma unroll
   for (int r = 0; r < MT; ++r) {
-    float v = wave_sum(acc[0][r]);
-    if (DUAL) v = silu_f(v) * wave_sum(acc[DUAL ? 1 : 0][r]);
+    const float v = wave_sum(acc[0][r]);
+    const float v2 = DUAL ? wave_sum(acc[DUAL ? 1 : 0][r]) : 0.f;
     if (lane == 0 && xr[r] >= 0) {
       const int64_t yrow = a.y_rows ? a.y_rows[m0 + r] : m0 + r;
-      a.y[yrow * a.ldy + n] = v * a.alpha;
+      a.y[yrow * a.ldy + n] = finish<DUAL>(a, yrow, n, v, v2);
     }
   }
 }
@@ -508,19 +527,47 @@ static int gemm_any_dispatch(const GemmAnyArgs& a, int w_dtype, int groups, int 
   return MI_EINVAL;
 }
 
+static bool act_ok(int act) { return act >= MI_ACT_NONE && act <= MI_ACT_SIGMOID; }
+
 extern "C" int mi_gemm_any(const float* x, int64_t ldx, const void* w, int w_dtype, float* y, int64_t ldy, int M, int N,
                            int K, float alpha, int exact, mi_stream stream) {
-  if (!x || !w || !y || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N) return MI_EINVAL;
-  GemmAnyArgs a{x, ldx, w, nullptr, y, ldy, M, N, K, alpha, nullptr, nullptr, nullptr};
+  return mi_gemm_any_act(x, ldx, w, nullptr, w_dtype, nullptr, nullptr, MI_ACT_NONE, y, ldy, M, N, K, alpha, exact, stream);
+}
+
+extern "C" int mi_gemm_any_act(const float* x, int64_t ldx, const void* w, const void* w2, int w_dtype, const float* bias,
+                               const float* bias2, int act, float* y, int64_t ldy, int M, int N, int K, float alpha,
+                               int exact, mi_stream stream) {
+  if (!x || !w || !y || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N || !act_ok(act) || (bias2 && !w2)) return MI_EINVAL;
+  GemmAnyArgs a{x, ldx, w, w2, y, ldy, M, N, K, alpha, nullptr, nullptr, nullptr, bias, bias2, act, nullptr, 0, 0, 0, 0};
   return gemm_any_dispatch(a, w_dtype, 1, M, exact ? 1 : 0, S(stream));
+}
+
+extern "C" int mi_gemm_any_batched(const float* x, int64_t ldx, int64_t x_batch, const void* w, int w_dtype, float* y,
+                                   int64_t ldy, int64_t y_batch, const float* gate, int64_t ldgate, int64_t gate_batch,
+                                   int n_batch, int M, int N, int K, int exact, mi_stream stream) {
+  if (!x || !w || !y || n_batch < 1 || M < 0 || N < 0 || K < 1 || ldx < K || ldy < N) return MI_EINVAL;
+  if (n_batch > 65535) return MI_EUNSUPPORTED;
+  GemmAnyArgs a{x, ldx, w, nullptr, y, ldy, M, N, K, 1.0f, nullptr, nullptr, nullptr, nullptr, nullptr, MI_ACT_NONE,
+                gate, ldgate, x_batch, y_batch, gate_batch};
+  return gemm_any_dispatch(a, w_dtype, n_batch, M, exact ? 1 : 0, S(stream));
 }
 
 extern "C" int mi_gemm_any_grouped(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2,
                                    int w_dtype, const int32_t* group_offsets, int n_groups, int rows_per_group_max,
                                    float* y, int64_t ldy, const int32_t* y_rows, int N, int K, int exact,
                                    mi_stream stream) {
-  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1) return MI_EINVAL;
+  return mi_gemm_any_grouped_act(x, ldx, x_rows, w, w2, w_dtype, w2 ? MI_ACT_SILU : MI_ACT_NONE, group_offsets, n_groups,
+                                 rows_per_group_max, y, ldy, y_rows, N, K, exact, stream);
+}
+
+extern "C" int mi_gemm_any_grouped_act(const float* x, int64_t ldx, const int32_t* x_rows, const void* w, const void* w2,
+                                       int w_dtype, int act, const int32_t* group_offsets, int n_groups,
+                                       int rows_per_group_max, float* y, int64_t ldy, const int32_t* y_rows, int N, int K,
+                                       int exact, mi_stream stream) {
+  if (!x || !w || !y || !group_offsets || n_groups < 1 || rows_per_group_max < 0 || N < 0 || K < 1 || !act_ok(act))
+    return MI_EINVAL;
   if (n_groups > 65535) return MI_EUNSUPPORTED;
-  GemmAnyArgs a{x, ldx, w, w2, y, ldy, rows_per_group_max, N, K, 1.0f, group_offsets, x_rows, y_rows};
+  GemmAnyArgs a{x, ldx, w, w2, y, ldy, rows_per_group_max, N, K, 1.0f, group_offsets, x_rows, y_rows, nullptr, nullptr,
+                act, nullptr, 0, 0, 0, 0};
   return gemm_any_dispatch(a, w_dtype, n_groups, rows_per_group_max, exact ? 1 : 0, S(stream));
 }

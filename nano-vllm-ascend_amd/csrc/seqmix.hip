@@ -136,6 +136,28 @@ __global__ __launch_bounds__(256) void swa_prepare_kernel(float* __restrict__ pr
   }
 }
 
+// Distance bias of a score, taken off it: kind MI_BIAS_SLOPE: 2^(-8 (h + 1) / H) * dist (p1 == nullptr) or p1[h] * dist;
+// MI_BIAS_LOG: p1[h] * ln(1 + p2[h] * dist); MI_BIAS_NONE: nothing.  ldv: elements between two tokens' value rows (Dv,
+// or the key row's length when the values are the leading channels of the key rows of the same cache).
+struct AttnBias {
+  int kind;
+  const float* p1;
+  const float* p2;
+};
+struct HeadBias {
+  float a, b;
+  bool log;
+};
+__device__ __forceinline__ HeadBias head_bias(const AttnBias& bias, int h, int H) {
+  HeadBias r{0.f, 0.f, bias.kind == MI_BIAS_LOG};
+  if (bias.kind == MI_BIAS_SLOPE) r.a = bias.p1 ? bias.p1[h] : exp2f(-8.f * (float)(h + 1) / (float)H);
+  else if (bias.kind == MI_BIAS_LOG) r.a = bias.p1[h], r.b = bias.p2[h];
+  return r;
+}
+__device__ __forceinline__ float dist_bias(const HeadBias& hb, int dist) {
+  return hb.log ? hb.a * log1pf(hb.b * (float)dist) : hb.a * (float)dist;
+}
+
 // The general form (any head sizes): one wave per (row, head); lanes over keys for the scores, over value channels for
 // the output, element-wise loads.
 template <typename TC, int VPL>  // VPL: value channels per lane (Dv <= 64 * VPL)
@@ -145,7 +167,8 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
                                                             const int32_t* __restrict__ cu_q,
                                                             const int32_t* __restrict__ kv_lens, int n_seqs, int n_rows,
                                                             int H, int G, int D, int Dv, int block_size, int window,
-                                                            float scale, const float* __restrict__ gate, int64_t ldg,
+                                                            float scale, AttnBias bias, int64_t ldv,
+                                                            const float* __restrict__ gate, int64_t ldg,
                                                             float* __restrict__ out, int64_t ldo) {
   extern __shared__ float smem[];  // per wave: q [D], p [64]
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -159,7 +182,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
   const int pos = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (row - cu_q[s]);
   const int lo = max(0, pos - window + 1);
   const int g = h / (H / G);
-  const float slope = exp2f(-8.f * (float)(h + 1) / (float)H);
+  const HeadBias hb = head_bias(bias, h, H);
   const int32_t* table = block_tables + (int64_t)s * table_cols;
   float m = -INFINITY, l = 0.f;
   float acc[VPL];
@@ -174,7 +197,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
       const TC* kr = k_cache + ((blk * G + g) * block_size + j % block_size) * D;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld_f<TC>(kr + d), dot);
-      sc = dot * scale - slope * (float)(pos - j);
+      sc = dot * scale - dist_bias(hb, pos - j);
     }
     const float m_new = fmaxf(m, wave_max(sc));
     const float p = j <= pos ? expf(sc - m_new) : 0.f;
@@ -189,7 +212,7 @@ __global__ __launch_bounds__(256) void swa_attention_kernel(const float* __restr
     for (int jj = 0; jj < n_keys; ++jj) {
       const int jk = j0 + jj;
       const int64_t blk = table[jk / block_size];
-      const TC* vr = v_cache + ((blk * G + g) * block_size + jk % block_size) * Dv;
+      const TC* vr = v_cache + ((blk * G + g) * block_size + jk % block_size) * ldv;
       const float pj = ps[jj];
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
@@ -243,8 +266,8 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
                                                                 const int32_t* __restrict__ cu_q,
                                                                 const int32_t* __restrict__ kv_lens, int n_seqs,
                                                                 int n_rows, int H, int G, int D, int Dv, int block_size,
-                                                                int window, float scale, int lpr_log2,
-                                                                const float* __restrict__ gate, int64_t ldg,
+                                                                int window, float scale, AttnBias bias, int64_t ldv,
+                                                                int lpr_log2, const float* __restrict__ gate, int64_t ldg,
                                                                 float* __restrict__ out, int64_t ldo) {
   static_assert(SPLIT == 1 || RPW == 1, "the split form is the single-row form");
   extern __shared__ float smem[];  // per wave: q [RPW][D], p [RPW][64]; SPLIT > 1: then per wave {m, l, acc [Dv]}
@@ -257,7 +280,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
   float* qs = smem + wave * RPW * (D + 64);
   float* ps = qs + RPW * D;
   const int g = h / (H / G);
-  const float slope = exp2f(-8.f * (float)(h + 1) / (float)H);
+  const HeadBias hb = head_bias(bias, h, H);
   const int lpr = 1 << lpr_log2, kg = lane >> lpr_log2, cg = lane & (lpr - 1), kpp = 64 >> lpr_log2;
   const int group_end = min(rg * RPW + RPW, n_rows);
   for (int first = rg * RPW; first < group_end;) {
@@ -304,7 +327,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
       for (int r = 0; r < RPW; ++r) {
         const int pos = pos0 + r;
         const bool vis = r < nr && j <= pos && j > pos - window;
-        const float sc = vis ? dots[r] * scale - slope * (float)(pos - j) : -INFINITY;
+        const float sc = vis ? dots[r] * scale - dist_bias(hb, pos - j) : -INFINITY;
         const float m_new = fmaxf(m[r], wave_max(sc));
         const float p = vis ? expf(sc - m_new) : 0.f;
         const float corr = m[r] == -INFINITY ? 0.f : expf(m[r] - m_new);
@@ -321,7 +344,7 @@ __global__ __launch_bounds__(256) void swa_attention_vec_kernel(const float* __r
           const int jk = j0 + jj;
           const int64_t blk = table[jk / block_size];
           float vv[VEC];
-          ld_vec<TC, VEC>(v_cache + ((blk * G + g) * block_size + jk % block_size) * Dv + cg * VEC, vv);
+          ld_vec<TC, VEC>(v_cache + ((blk * G + g) * block_size + jk % block_size) * ldv + cg * VEC, vv);
 #pragma unroll
           for (int r = 0; r < RPW; ++r) {
             const float pj = ps[r * 64 + jj];
@@ -395,15 +418,16 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
                                                                  const int32_t* __restrict__ cu_q,
                                                                  const int32_t* __restrict__ kv_lens, int n_seqs,
                                                                  int n_rows, int H, int G, int D, int Dv, int block_size,
-                                                                 int window, float scale, const float* __restrict__ gate,
-                                                                 int64_t ldg, float* __restrict__ out, int64_t ldo) {
+                                                                 int window, float scale, AttnBias bias, int64_t ldv,
+                                                                 const float* __restrict__ gate, int64_t ldg,
+                                                                 float* __restrict__ out, int64_t ldo) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wid = blockIdx.x * 4 + wave;
   const int n_groups = (n_rows + 15) / 16;
   if (wid >= n_groups * H) return;
   const int rg = wid / H, h = wid % H;
   const int g = h / (H / G);
-  const float slope = exp2f(-8.f * (float)(h + 1) / (float)H);
+  const HeadBias hb = head_bias(bias, h, H);
   const int qi = lane & 15, kg = lane >> 4;
   const int dk = D / 32, dvt = Dv / 16;
   const bool q_vec = (ldq % 4 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15u) == 0) && (D % 4 == 0);
@@ -465,7 +489,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
       for (int e = 0; e < 8; ++e) {
         const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
         vis[e] = qi < nr && key <= my_pos && key > my_pos - window;
-        sc[e] = vis[e] ? sacc[e >> 2][e & 3] * scale - slope * (float)(my_pos - key) : -INFINITY;
+        sc[e] = vis[e] ? sacc[e >> 2][e & 3] * scale - dist_bias(hb, my_pos - key) : -INFINITY;
         mx = fmaxf(mx, sc[e]);
       }
       mx = xor_max<32>(xor_max<16>(mx));
@@ -493,7 +517,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
       for (int e = 0; e < 8; ++e) {
         const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
         vrow[e] = key <= hi_key
-                      ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * Dv +
+                      ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
                             (PAIR ? 2 * qi : qi)
                       : nullptr;
       }
@@ -887,6 +911,311 @@ __global__ __launch_bounds__(256) void moe_combine_f32_kernel(const float* __res
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// pre-norm residual streams: RMS norm, residual update, depth-weighted mixing of the layers' results
+// ---------------------------------------------------------------------------------------------------------------
+// One workgroup per row.  res += mult * y (y may be nullptr); w != nullptr: out = res / sqrt(mean(res^2) + eps) * (w + shift)
+// (shift 1: weights stored around zero).  res == out is allowed (a plain norm in place).
+__global__ __launch_bounds__(256) void add_rmsnorm_f32_kernel(float* __restrict__ res, int64_t ldr,
+                                                              const float* __restrict__ y, int64_t ldy, float mult,
+                                                              const float* __restrict__ w, float shift, float eps,
+                                                              float* __restrict__ out, int64_t ldo, int width) {
+  __shared__ float red[4];
+  float* r = res + (int64_t)blockIdx.x * ldr;
+  const float* yr = y ? y + (int64_t)blockIdx.x * ldy : nullptr;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float v = r[c];
+    if (yr) {
+      v = fmaf(mult, yr[c], v);
+      r[c] = v;
+    }
+    sq = fmaf(v, v, sq);
+  }
+  if (!w) return;
+  const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)width + eps);
+  float* o = out + (int64_t)blockIdx.x * ldo;
+  for (int c = threadIdx.x; c < width; c += 256) o[c] = r[c] * rstd * (w[c] + shift);  // (a thread re-reads its own writes)
+}
+
+// The results X_0 .. X_{n-1} of the embedding and of the layers so far are the slots of one buffer (slot_stride floats
+// apart).  X_{n-1} += mult * y (the last sublayer's output, may be nullptr); slot n <- sum_j coef[j] X_j; norm_w != nullptr:
+// h = slot n / rms * (norm_w + shift) - what the next layer's mixer reads.
+__global__ __launch_bounds__(256) void depth_mix_f32_kernel(float* __restrict__ stack, int64_t slot_stride, int n,
+                                                            const float* __restrict__ coef, const float* __restrict__ y,
+                                                            int64_t ldy, float mult, const float* __restrict__ norm_w,
+                                                            float shift, float eps, float* __restrict__ h, int64_t ldh,
+                                                            int width) {
+  __shared__ float red[4];
+  float* base = stack + (int64_t)blockIdx.x * width;
+  float* last = base + (int64_t)(n - 1) * slot_stride;
+  float* dst = base + (int64_t)n * slot_stride;
+  const float* yr = y ? y + (int64_t)blockIdx.x * ldy : nullptr;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float xl = last[c];
+    if (yr) {
+      xl = fmaf(mult, yr[c], xl);
+      last[c] = xl;
+    }
+    float acc = 0.f;
+    for (int j = 0; j + 1 < n; ++j) acc = fmaf(coef[j], base[(int64_t)j * slot_stride + c], acc);
+    acc = fmaf(coef[n - 1], xl, acc);
+    dst[c] = acc;
+    sq = fmaf(acc, acc, sq);
+  }
+  if (!norm_w) return;
+  const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)width + eps);
+  float* o = h + (int64_t)blockIdx.x * ldh;
+  for (int c = threadIdx.x; c < width; c += 256) o[c] = dst[c] * rstd * (norm_w[c] + shift);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// minimal gated recurrence: S_p = (1 - z_p) S_{p-1} + z_p c_p per channel, out = S_p * silu(g_p)
+// ---------------------------------------------------------------------------------------------------------------
+// z = sigmoid(zp), c = up + 1/2 (up >= 0) | sigmoid(up) (up < 0); zp, up, gp are columns of one projection buffer.
+// The recurrence is linear in S, so a sequence's rows of this step are cut into segments of kScanSeg rows that are
+// walked in parallel: (1) every segment but a sequence's last computes its (A, B) with S_end = A S_start + B;
+// (2) one thread per (sequence, channel) turns them into every segment's S_start, beginning with the slot's state (zero
+// when the sequence starts in this step); (3) every segment walks its rows from its S_start and writes the outputs, a
+// sequence's last segment also the slot's new state.  A step whose sequences all fit one segment (decode steps, short
+// portions) is launch (3) alone.
+constexpr int kScanSeg = 64;
+
+struct ScanSeg {
+  int s, first, count, index, total;  // sequence, first step row, rows, segment index within the sequence, its segments
+};
+// segment `id` of the step (segments are numbered sequence by sequence); count = 0: beyond the last one
+__device__ __forceinline__ ScanSeg scan_segment(const int32_t* cu_q, int n_seqs, int id) {
+  ScanSeg r{0, 0, 0, 0, 0};
+  for (int s = 0; s < n_seqs; ++s) {
+    const int n = cu_q[s + 1] - cu_q[s];
+    const int segs = (n + kScanSeg - 1) / kScanSeg;
+    if (id < segs) {
+      r.s = s, r.index = id, r.total = segs;
+      r.first = cu_q[s] + id * kScanSeg;
+      r.count = min(kScanSeg, n - id * kScanSeg);
+      return r;
+    }
+    id -= segs;
+  }
+  return r;
+}
+__device__ __forceinline__ void mingru_gates(float zp, float up, float& keep, float& add) {
+  const float z = sigmoid_f(zp);
+  const float c = up >= 0.f ? up + 0.5f : sigmoid_f(up);
+  keep = 1.f - z;
+  add = z * c;
+}
+
+__global__ __launch_bounds__(256) void mingru_summary_kernel(const float* __restrict__ proj, int64_t ld, int z_off,
+                                                             int x_off, const int32_t* __restrict__ cu_q, int n_seqs,
+                                                             int width, float* __restrict__ summary) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const ScanSeg sg = scan_segment(cu_q, n_seqs, blockIdx.y);
+  if (c >= width || sg.count == 0 || sg.index + 1 == sg.total) return;
+  float A = 1.f, B = 0.f;
+  for (int r = 0; r < sg.count; ++r) {
+    const float* row = proj + (int64_t)(sg.first + r) * ld;
+    float keep, add;
+    mingru_gates(row[z_off + c], row[x_off + c], keep, add);
+    A *= keep;
+    B = fmaf(keep, B, add);
+  }
+  summary[((int64_t)blockIdx.y * 2) * width + c] = A;
+  summary[((int64_t)blockIdx.y * 2 + 1) * width + c] = B;
+}
+
+// S_start of every segment, written over the segment's A (segment 0 of a sequence: the carried state)
+__global__ __launch_bounds__(256) void mingru_carry_kernel(float* __restrict__ summary, const float* __restrict__ state,
+                                                           const int32_t* __restrict__ cu_q,
+                                                           const int32_t* __restrict__ kv_lens,
+                                                           const int32_t* __restrict__ slot_ids, int width) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int n = cu_q[s + 1] - cu_q[s];
+  if (n == 0) return;
+  int id0 = 0;
+  for (int t = 0; t < s; ++t) id0 += (cu_q[t + 1] - cu_q[t] + kScanSeg - 1) / kScanSeg;
+  const int segs = (n + kScanSeg - 1) / kScanSeg;
+  float S = kv_lens[s] - n > 0 ? state[(int64_t)slot_ids[s] * width + c] : 0.f;
+  for (int k = 0; k < segs; ++k) {
+    float* e = summary + ((int64_t)(id0 + k) * 2) * width + c;
+    const float A = e[0], B = e[width];
+    e[0] = S;
+    if (k + 1 < segs) S = fmaf(A, S, B);
+  }
+}
+
+template <bool CARRIED>  // CARRIED: S_start from the summary buffer; else every sequence is one segment: from the slot
+__global__ __launch_bounds__(256) void mingru_walk_kernel(const float* __restrict__ proj, int64_t ld, int z_off, int x_off,
+                                                          int g_off, const float* __restrict__ summary,
+                                                          float* __restrict__ state, const int32_t* __restrict__ cu_q,
+                                                          const int32_t* __restrict__ kv_lens,
+                                                          const int32_t* __restrict__ slot_ids, int n_seqs, int width,
+                                                          float* __restrict__ out, int64_t ldo) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const ScanSeg sg = scan_segment(cu_q, n_seqs, blockIdx.y);
+  if (c >= width || sg.count == 0) return;
+  float S;
+  if (CARRIED) S = summary[((int64_t)blockIdx.y * 2) * width + c];
+  else S = kv_lens[sg.s] - (cu_q[sg.s + 1] - cu_q[sg.s]) > 0 ? state[(int64_t)slot_ids[sg.s] * width + c] : 0.f;
+  for (int r = 0; r < sg.count; ++r) {
+    const float* row = proj + (int64_t)(sg.first + r) * ld;
+    float keep, add;
+    mingru_gates(row[z_off + c], row[x_off + c], keep, add);
+    S = fmaf(keep, S, add);
+    const float g = row[g_off + c];
+    out[(int64_t)(sg.first + r) * ldo + c] = S * (g / (1.f + expf(-g)));
+  }
+  if (sg.index + 1 == sg.total) state[(int64_t)slot_ids[sg.s] * width + c] = S;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// per-row preparation of the paged attentions without a whole-projection norm
+// ---------------------------------------------------------------------------------------------------------------
+// Plain grouped heads: q <- q * (1 + coef * ln(floor((p + 1) / every) + 1)) in place (every < 1: no temperature), k and
+// v rows to the cache.  One workgroup per row.
+template <typename TC>
+__global__ __launch_bounds__(256) void kv_store_temp_kernel(float* __restrict__ proj, int64_t ld, int q_off, int k_off,
+                                                            int v_off, int nq, float coef, int every,
+                                                            const int32_t* __restrict__ cu_q,
+                                                            const int32_t* __restrict__ kv_lens, int n_seqs,
+                                                            TC* __restrict__ k_cache, TC* __restrict__ v_cache,
+                                                            const int32_t* __restrict__ slots, int G, int D, int Dv,
+                                                            int block_size) {
+  const int row = blockIdx.x;
+  float* r = proj + (int64_t)row * ld;
+  if (every >= 1) {
+    const int s = seq_of_row(cu_q, n_seqs, row);
+    const int pos = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (row - cu_q[s]);
+    const float temp = 1.f + coef * logf((float)((pos + 1) / every) + 1.f);
+    for (int c = threadIdx.x; c < nq; c += 256) r[q_off + c] *= temp;
+  }
+  const int slot = slots[row];
+  if (slot < 0) return;
+  const int64_t blk = slot / block_size;
+  const int off = slot % block_size;
+  for (int c = threadIdx.x; c < G * D; c += 256)
+    st_f<TC>(k_cache + ((blk * G + c / D) * block_size + off) * D + c % D, r[k_off + c]);
+  for (int c = threadIdx.x; c < G * Dv; c += 256)
+    st_f<TC>(v_cache + ((blk * G + c / Dv) * block_size + off) * Dv + c % Dv, r[v_off + c]);
+}
+
+// Latent attention: the row's compressed key/value c (C entries at c_off) is RMS-normed with a plain weight and stored as
+// the leading C channels of the row's cache entry, the shared rotated key part (R entries behind it) is rotated by the
+// row's position and stored behind them: a cache row is [c | r], one "kv head" that every query head reads, keys = the
+// whole row, values = its first C channels.  The rotated part of every query head (R entries at q_off + h * (D + R) + D)
+// is rotated and written to qx[row][h][C ..] - the head's absorbed key-space query [W_uk^T q | rot(q_r)] whose first C
+// entries a batched projection fills in.  Rotation: the first `dims` entries, pairs (i, i + dims / 2), angle
+// pos * base^(-2 i / dims), computed in fp32 (powf / sincosf of the device library).
+template <typename TC>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __restrict__ proj, int64_t ld, int q_off,
+                                                             int c_off, int H, int D, int R, int C, int dims, float base,
+                                                             const float* __restrict__ norm_w, float eps,
+                                                             const int32_t* __restrict__ cu_q,
+                                                             const int32_t* __restrict__ kv_lens, int n_seqs,
+                                                             TC* __restrict__ cache, const int32_t* __restrict__ slots,
+                                                             float* __restrict__ qx, int64_t ldqx) {
+  __shared__ float red[4];
+  const int row = blockIdx.x;
+  const float* r = proj + (int64_t)row * ld;
+  const int s = seq_of_row(cu_q, n_seqs, row);
+  const int pos = kv_lens[s] - (cu_q[s + 1] - cu_q[s]) + (row - cu_q[s]);
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < C; c += 256) sq = fmaf(r[c_off + c], r[c_off + c], sq);
+  const float rstd = 1.f / sqrtf(block_sum256(sq, red) / (float)C + eps);
+  const int slot = slots[row];
+  TC* dst = slot >= 0 ? cache + (int64_t)slot * (C + R) : nullptr;
+  if (dst)
+    for (int c = threadIdx.x; c < C; c += 256) st_f<TC>(dst + c, r[c_off + c] * rstd * norm_w[c]);
+  const int half = dims / 2;
+  // unit u = 0: the shared key part; u = 1 + h: query head h
+  for (int i = threadIdx.x; i < (H + 1) * R; i += 256) {
+    const int u = i / R, e = i % R;
+    const float* src = u == 0 ? r + c_off + C : r + q_off + (int64_t)(u - 1) * (D + R) + D;
+    float v = src[e];
+    if (e < dims) {
+      const int f = e < half ? e : e - half;
+      const float ang = (float)pos * powf(base, -2.f * (float)f / (float)dims);
+      float sn, cs;
+      sincosf(ang, &sn, &cs);
+      v = e < half ? src[e] * cs - src[e + half] * sn : src[e] * cs + src[e - half] * sn;
+    }
+    if (u == 0) {
+      if (dst) st_f<TC>(dst + C + e, v);
+    } else {
+      qx[(int64_t)row * ldqx + (int64_t)(u - 1) * (C + R) + C + e] = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// plain top-k router: the top_k largest logits (equal values: the lower index), weights = softmax over the chosen
+// ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, int64_t ld, int T, int n,
+                                                         int top_k, int32_t* __restrict__ ids, float* __restrict__ wts) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  const float* z = logits + (int64_t)t * ld;
+  constexpr int EPL = 8;
+  const int big = 1 << 30;
+  float sc[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    sc[i] = e < n ? z[e] : -INFINITY;
+    if (!(sc[i] == sc[i])) sc[i] = -INFINITY;
+  }
+  unsigned taken = 0;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i)
+    if (lane + 64 * i >= n) taken |= 1u << i;
+  float top = 0.f, sum = 0.f;
+  float mine[EPL];  // exp(logit - top) of the outputs this lane gave away, in pick order
+  int my_slot[EPL], n_mine = 0;
+  for (int it = 0; it < top_k; ++it) {
+    float bv = -INFINITY;
+    int bi = big;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (!(taken >> i & 1) && (bi == big || sc[i] > bv)) bv = sc[i], bi = lane + 64 * i;
+    wave_argmax(bv, bi);
+    if (it == 0) top = bv;
+    const float p = expf(bv - top);
+    sum += p;
+    if ((bi & 63) == lane) {
+      taken |= 1u << (bi >> 6);
+      ids[(int64_t)t * top_k + it] = bi;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i)
+        if (i == n_mine) mine[i] = p, my_slot[i] = it;
+      ++n_mine;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < EPL; ++i)
+    if (i < n_mine) wts[(int64_t)t * top_k + my_slot[i]] = mine[i] / sum;
+}
+
+// out[t] = sum_k w[t][k] y[t * top_k + k] + sigmoid(shared_gate[t]) * shared[t]   (shared == nullptr: no shared part)
+__global__ __launch_bounds__(256) void moe_combine_shared_kernel(const float* __restrict__ y, const int32_t* __restrict__ ids,
+                                                                 const float* __restrict__ wts, int top_k, int width,
+                                                                 const float* __restrict__ shared, int64_t lds_,
+                                                                 const float* __restrict__ shared_gate, int64_t ldsg,
+                                                                 float* __restrict__ out, int64_t ldo) {
+  const int t = blockIdx.x;
+  const float sgate = shared ? sigmoid_f(shared_gate[(int64_t)t * ldsg]) : 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float acc = 0.f;
+    for (int k = 0; k < top_k; ++k) acc = fmaf(wts[(int64_t)t * top_k + k], y[((int64_t)t * top_k + k) * width + c], acc);
+    if (shared) acc = fmaf(sgate, shared[(int64_t)t * lds_ + c], acc);
+    out[(int64_t)t * ldo + c] = acc;
+  }
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -936,18 +1265,18 @@ extern "C" int mi_swa_prepare(float* proj, int64_t ld, int q_off, int k_off, int
 template <typename TC>
 static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* vc, const int32_t* bt, int cols,
                       const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
-                      int block_size, int window, float scale, const float* gate, int64_t ldg, float* out, int64_t ldo,
-                      hipStream_t st) {
+                      int block_size, int window, float scale, AttnBias bias, int64_t ldv, const float* gate, int64_t ldg,
+                      float* out, int64_t ldo, hipStream_t st) {
   const TC* k = static_cast<const TC*>(kc);
   const TC* v = static_cast<const TC*>(vc);
   constexpr int VEC = 16 / sizeof(TC);
   if constexpr (sizeof(TC) == 2) {
     // prompt portions over a bf16 cache: the matrix-core form
-    if (rows > n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256) {
+    if (rows > n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0) {
       const dim3 grid_m((((rows + 15) / 16) * H + 3) / 4);
 #define MI_SWA_MFMA(DKM, DVM, PAIR)                                                                                    \
   hipLaunchKernelGGL((swa_attention_mfma_kernel<DKM, DVM, PAIR>), grid_m, dim3(256), 0, st, q, ldq, k, v, bt, cols, cu_q, \
-                     kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo)
+                     kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo)
       const bool small = D <= 128 && Dv <= 128, pair = Dv % 32 == 0;
       if (small && pair) MI_SWA_MFMA(4, 8, true);
       else if (small) MI_SWA_MFMA(4, 8, false);
@@ -957,7 +1286,7 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
       return check_launch();
     }
   }
-  if (D % VEC == 0 && Dv % VEC == 0 && Dv / VEC <= 64) {
+  if (D % VEC == 0 && Dv % VEC == 0 && Dv / VEC <= 64 && ldv % VEC == 0) {
     int lpr_log2 = 0;
     while ((1 << lpr_log2) * VEC < Dv) ++lpr_log2;
     // rows == n_seqs: every sequence brings one row (a decode step): a wave per row; else four rows per wave
@@ -967,11 +1296,11 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
       if (rpw == 4)
         hipLaunchKernelGGL((swa_attention_vec_kernel<TC, VEC, 4, 1>), dim3((((rows + 3) / 4) * H + 3) / 4), dim3(256),
                            lds_v, st, q, ldq, k, v, bt, cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window,
-                           scale, lpr_log2, gate, ldg, out, ldo);
+                           scale, bias, ldv, lpr_log2, gate, ldg, out, ldo);
       else
         hipLaunchKernelGGL((swa_attention_vec_kernel<TC, VEC, 1, 4>), dim3(rows * H), dim3(256), lds_v, st, q, ldq, k, v,
-                           bt, cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window, scale, lpr_log2, gate,
-                           ldg, out, ldo);
+                           bt, cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv, block_size, window, scale, bias, ldv, lpr_log2,
+                           gate, ldg, out, ldo);
       return check_launch();
     }
   }
@@ -980,10 +1309,11 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
   if (lds > 48 * 1024) return MI_EUNSUPPORTED;
 #define MI_SWA(VPL)                                                                                                  \
   hipLaunchKernelGGL((swa_attention_kernel<TC, VPL>), grid, block, lds, st, q, ldq, k, v, bt, cols, cu_q, kv_lens,     \
-                     n_seqs, rows, H, G, D, Dv, block_size, window, scale, gate, ldg, out, ldo)
+                     n_seqs, rows, H, G, D, Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo)
   if (Dv <= 64) MI_SWA(1);
   else if (Dv <= 128) MI_SWA(2);
-  else MI_SWA(4);
+  else if (Dv <= 256) MI_SWA(4);
+  else MI_SWA(8);
 #undef MI_SWA
   return check_launch();
 }
@@ -992,16 +1322,30 @@ extern "C" int mi_swa_attention(const float* q, int64_t ldq, const void* k_cache
                                 const int32_t* block_tables, int table_cols, const int32_t* cu_q, const int32_t* kv_lens,
                                 int n_seqs, int rows, int H, int G, int D, int Dv, int block_size, int window,
                                 float scale, const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream) {
+  return mi_paged_attention_f32(q, ldq, k_cache, v_cache, Dv, cache_dtype, block_tables, table_cols, cu_q, kv_lens, n_seqs,
+                                rows, H, G, D, Dv, block_size, window, scale, MI_BIAS_SLOPE, nullptr, nullptr, gate, ldg,
+                                out, ldo, stream);
+}
+
+extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
+                                      int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
+                                      const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
+                                      int block_size, int window, float scale, int bias_kind, const float* bias_p1,
+                                      const float* bias_p2, const float* gate, int64_t ldg, float* out, int64_t ldo,
+                                      mi_stream stream) {
   if (!q || !k_cache || !v_cache || !block_tables || !cu_q || !kv_lens || !out || rows < 0 || n_seqs < 1) return MI_EINVAL;
-  if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1 || block_size < 1 || window < 1 || table_cols < 1) return MI_EINVAL;
-  if (Dv > 256 || D > 4096) return MI_EUNSUPPORTED;
+  if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1 || block_size < 1 || window < 1 || table_cols < 1 || ldv < Dv) return MI_EINVAL;
+  if (bias_kind != MI_BIAS_SLOPE && bias_kind != MI_BIAS_LOG && bias_kind != MI_BIAS_NONE) return MI_EINVAL;
+  if (bias_kind == MI_BIAS_LOG && (!bias_p1 || !bias_p2)) return MI_EINVAL;
+  if (Dv > 512 || D > 4096) return MI_EUNSUPPORTED;
   if (rows == 0) return MI_OK;
+  const AttnBias bias{bias_kind, bias_p1, bias_p2};
   if (cache_dtype == MI_DTYPE_BF16)
     return launch_swa<uint16_t>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D,
-                                Dv, block_size, window, scale, gate, ldg, out, ldo, S(stream));
+                                Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo, S(stream));
   if (cache_dtype == MI_DTYPE_F32)
     return launch_swa<float>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv,
-                             block_size, window, scale, gate, ldg, out, ldo, S(stream));
+                             block_size, window, scale, bias, ldv, gate, ldg, out, ldo, S(stream));
   return MI_EINVAL;
 }
 
@@ -1089,5 +1433,116 @@ extern "C" int mi_moe_combine_f32(const float* y, const float* h, int64_t ldh, c
   if (n_tokens == 0) return MI_OK;
   hipLaunchKernelGGL(moe_combine_f32_kernel, dim3(n_tokens), dim3(256), 0, S(stream), y, h, ldh, ids, weights, top_k,
                      n_experts, width, out, ldo);
+  return check_launch();
+}
+
+extern "C" int mi_add_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* w,
+                                  float shift, float eps, float* out, int64_t ldo, int rows, int width, mi_stream stream) {
+  if (!res || rows < 0 || width < 1 || ldr < width || (y && ldy < width) || (w && (!out || ldo < width))) return MI_EINVAL;
+  if (rows == 0 || (!y && !w)) return MI_OK;
+  hipLaunchKernelGGL(add_rmsnorm_f32_kernel, dim3(rows), dim3(256), 0, S(stream), res, ldr, y, ldy, mult, w, shift, eps, out,
+                     ldo, width);
+  return check_launch();
+}
+
+extern "C" int mi_depth_mix_f32(float* stack, int64_t slot_stride, int n, const float* coef, const float* y, int64_t ldy,
+                                float mult, const float* norm_w, float shift, float eps, float* h, int64_t ldh, int rows,
+                                int width, mi_stream stream) {
+  if (!stack || !coef || n < 1 || rows < 0 || width < 1 || slot_stride < (int64_t)rows * width) return MI_EINVAL;
+  if ((y && ldy < width) || (norm_w && (!h || ldh < width))) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  hipLaunchKernelGGL(depth_mix_f32_kernel, dim3(rows), dim3(256), 0, S(stream), stack, slot_stride, n, coef, y, ldy, mult,
+                     norm_w, shift, eps, h, ldh, width);
+  return check_launch();
+}
+
+extern "C" int64_t mi_mingru_scan_workspace_elems(int rows, int n_seqs, int width) {
+  if (rows < 0 || n_seqs < 1 || width < 1) return -1;
+  return 2 * (int64_t)(rows / kScanSeg + n_seqs) * width;
+}
+
+extern "C" int mi_mingru_scan(const float* proj, int64_t ld, int z_off, int x_off, int g_off, float* state,
+                              const int32_t* cu_q, const int32_t* kv_lens, const int32_t* slot_ids, int n_seqs, int rows,
+                              int max_rows_per_seq, int width, float* workspace, float* out, int64_t ldo,
+                              mi_stream stream) {
+  if (!proj || !state || !cu_q || !kv_lens || !slot_ids || !out || n_seqs < 1 || rows < 0 || width < 1) return MI_EINVAL;
+  if (z_off < 0 || x_off < 0 || g_off < 0 || ld < width || ldo < width || max_rows_per_seq < 1) return MI_EINVAL;
+  if (n_seqs > 65535) return MI_EUNSUPPORTED;
+  if (rows == 0) return MI_OK;
+  const int cb = (width + 255) / 256;
+  const int max_segs = rows / kScanSeg + n_seqs;  // (sum over the sequences of ceil(rows_s / seg) is at most this)
+  if (max_rows_per_seq <= kScanSeg) {
+    hipLaunchKernelGGL((mingru_walk_kernel<false>), dim3(cb, n_seqs), dim3(256), 0, S(stream), proj, ld, z_off, x_off, g_off,
+                       (const float*)nullptr, state, cu_q, kv_lens, slot_ids, n_seqs, width, out, ldo);
+    return check_launch();
+  }
+  if (!workspace || max_segs > 65535) return !workspace ? MI_EINVAL : MI_EUNSUPPORTED;
+  hipLaunchKernelGGL(mingru_summary_kernel, dim3(cb, max_segs), dim3(256), 0, S(stream), proj, ld, z_off, x_off, cu_q,
+                     n_seqs, width, workspace);
+  if (check_launch() != MI_OK) return MI_ELAUNCH;
+  hipLaunchKernelGGL(mingru_carry_kernel, dim3(cb, n_seqs), dim3(256), 0, S(stream), workspace, state, cu_q, kv_lens,
+                     slot_ids, width);
+  if (check_launch() != MI_OK) return MI_ELAUNCH;
+  hipLaunchKernelGGL((mingru_walk_kernel<true>), dim3(cb, max_segs), dim3(256), 0, S(stream), proj, ld, z_off, x_off, g_off,
+                     workspace, state, cu_q, kv_lens, slot_ids, n_seqs, width, out, ldo);
+  return check_launch();
+}
+
+extern "C" int mi_kv_store_temp(float* proj, int64_t ld, int q_off, int k_off, int v_off, float temp_coef, int temp_every,
+                                const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, void* k_cache, void* v_cache,
+                                int cache_dtype, const int32_t* slots, int rows, int H, int G, int D, int Dv,
+                                int block_size, mi_stream stream) {
+  if (!proj || !cu_q || !kv_lens || !k_cache || !v_cache || !slots || rows < 0 || n_seqs < 1) return MI_EINVAL;
+  if (H < 1 || G < 1 || D < 1 || Dv < 1 || block_size < 1) return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  if (cache_dtype == MI_DTYPE_BF16)
+    hipLaunchKernelGGL((kv_store_temp_kernel<uint16_t>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, k_off, v_off,
+                       H * D, temp_coef, temp_every, cu_q, kv_lens, n_seqs, static_cast<uint16_t*>(k_cache),
+                       static_cast<uint16_t*>(v_cache), slots, G, D, Dv, block_size);
+  else if (cache_dtype == MI_DTYPE_F32)
+    hipLaunchKernelGGL((kv_store_temp_kernel<float>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, k_off, v_off,
+                       H * D, temp_coef, temp_every, cu_q, kv_lens, n_seqs, static_cast<float*>(k_cache),
+                       static_cast<float*>(v_cache), slots, G, D, Dv, block_size);
+  else return MI_EINVAL;
+  return check_launch();
+}
+
+extern "C" int mi_latent_prepare(const float* proj, int64_t ld, int q_off, int c_off, int H, int D, int R, int C,
+                                 int rot_dims, float rot_base, const float* norm_w, float eps, const int32_t* cu_q,
+                                 const int32_t* kv_lens, int n_seqs, void* cache, int cache_dtype, const int32_t* slots,
+                                 float* qx, int64_t ldqx, int rows, mi_stream stream) {
+  if (!proj || !norm_w || !cu_q || !kv_lens || !cache || !slots || !qx || rows < 0 || n_seqs < 1) return MI_EINVAL;
+  if (H < 1 || D < 0 || R < 0 || C < 1 || rot_dims < 0 || rot_dims > R || rot_dims % 2 || ldqx < (int64_t)H * (C + R))
+    return MI_EINVAL;
+  if (rows == 0) return MI_OK;
+  if (cache_dtype == MI_DTYPE_BF16)
+    hipLaunchKernelGGL((latent_prepare_kernel<uint16_t>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, c_off, H, D,
+                       R, C, rot_dims, rot_base, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<uint16_t*>(cache), slots,
+                       qx, ldqx);
+  else if (cache_dtype == MI_DTYPE_F32)
+    hipLaunchKernelGGL((latent_prepare_kernel<float>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, c_off, H, D, R,
+                       C, rot_dims, rot_base, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<float*>(cache), slots, qx,
+                       ldqx);
+  else return MI_EINVAL;
+  return check_launch();
+}
+
+extern "C" int mi_route_topk(const float* logits, int64_t ld, int n_tokens, int n_outputs, int top_k, int32_t* ids,
+                             float* weights, mi_stream stream) {
+  if (!logits || !ids || !weights || n_tokens < 0 || ld < n_outputs) return MI_EINVAL;
+  if (n_outputs < 1 || n_outputs > 512 || top_k < 1 || top_k > n_outputs) return MI_EUNSUPPORTED;
+  if (n_tokens == 0) return MI_OK;
+  hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, S(stream), logits, ld, n_tokens, n_outputs,
+                     top_k, ids, weights);
+  return check_launch();
+}
+
+extern "C" int mi_moe_combine_shared(const float* y, const int32_t* ids, const float* weights, int n_tokens, int top_k,
+                                     int width, const float* shared, int64_t ld_shared, const float* shared_gate,
+                                     int64_t ld_gate, float* out, int64_t ldo, mi_stream stream) {
+  if (!y || !ids || !weights || !out || n_tokens < 0 || top_k < 1 || width < 1 || (shared && !shared_gate)) return MI_EINVAL;
+  if (n_tokens == 0) return MI_OK;
+  hipLaunchKernelGGL(moe_combine_shared_kernel, dim3(n_tokens), dim3(256), 0, S(stream), y, ids, weights, top_k, width,
+                     shared, ld_shared, shared_gate, ld_gate, out, ldo);
   return check_launch();
 }

@@ -25,6 +25,8 @@ LIB_PATH = os.environ.get(
 MI_OK = 0
 MI_EUNSUPPORTED = -2
 DTYPE_BF16, DTYPE_F32 = 0, 1
+ACT_NONE, ACT_SILU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_SIGMOID = range(5)   # MI_ACT_*
+BIAS_SLOPE, BIAS_LOG, BIAS_NONE = range(3)                                # MI_BIAS_*
 HEAD_DIM = 128
 KV_TILE_TOKENS = 16
 KV_TILE_ELEMS = 2048
@@ -181,6 +183,26 @@ _SIGNATURES = {
                                  _p, _p, _p, _p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, _p, c_int64, _p]),
     "mi_route_grouped": (c_int, [_p, c_int64, _p, c_int, c_int, c_int, c_int, c_int, _p, _p, _p]),
     "mi_moe_combine_f32": (c_int, [_p, _p, c_int64, _p, _p, c_int, c_int, c_int, c_int, _p, c_int64, _p]),
+    "mi_gemm_any_act": (c_int, [_p, c_int64, _p, _p, c_int, _p, _p, c_int, _p, c_int64, c_int, c_int, c_int, c_float,
+                                c_int, _p]),
+    "mi_gemm_any_grouped_act": (c_int, [_p, c_int64, _p, _p, _p, c_int, c_int, _p, c_int, c_int, _p, c_int64, _p, c_int,
+                                        c_int, c_int, _p]),
+    "mi_gemm_any_batched": (c_int, [_p, c_int64, c_int64, _p, c_int, _p, c_int64, c_int64, _p, c_int64, c_int64, c_int,
+                                    c_int, c_int, c_int, c_int, _p]),
+    "mi_paged_attention_f32": (c_int, [_p, c_int64, _p, _p, c_int64, c_int, _p, c_int, _p, _p, c_int, c_int, c_int, c_int,
+                                       c_int, c_int, c_int, c_int, c_float, c_int, _p, _p, _p, c_int64, _p, c_int64, _p]),
+    "mi_add_rmsnorm_f32": (c_int, [_p, c_int64, _p, c_int64, c_float, _p, c_float, c_float, _p, c_int64, c_int, c_int, _p]),
+    "mi_depth_mix_f32": (c_int, [_p, c_int64, c_int, _p, _p, c_int64, c_float, _p, c_float, c_float, _p, c_int64, c_int,
+                                 c_int, _p]),
+    "mi_mingru_scan_workspace_elems": (c_int64, [c_int, c_int, c_int]),
+    "mi_mingru_scan": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, _p, _p, _p, c_int, c_int, c_int, c_int, _p, _p,
+                               c_int64, _p]),
+    "mi_kv_store_temp": (c_int, [_p, c_int64, c_int, c_int, c_int, c_float, c_int, _p, _p, c_int, _p, _p, c_int, _p, c_int,
+                                 c_int, c_int, c_int, c_int, c_int, _p]),
+    "mi_latent_prepare": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_float, _p,
+                                  _p, c_int, _p, c_int, _p, _p, c_int64, c_int, _p]),
+    "mi_route_topk": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, _p, _p]),
+    "mi_moe_combine_shared": (c_int, [_p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p, c_int64, _p, c_int64, _p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -10,6 +10,16 @@ configuration:
                             recurrent state and convolution tail live in per-sequence state slots
   GroupedSparseMLP          sparse mixture of SwiGLU experts, group-limited top-k routing with a choice correction,
                             un-renormalised weights, identity experts
+  DepthMixedResidual        pre-norm residual stream x <- x + m f(norm(x)) whose layers read a learned weighted sum of the
+                            embedding and of all earlier layers' results; RMS norms with weights stored around zero
+  MinGRUMixer               minimal gated recurrence (gates from the current token only), fp32 state per sequence slot
+  LatentAttention           attention over a low-rank key/value latent plus one shared rotated key part; only those are
+                            cached, the per-head up-projections are absorbed into the query and the output
+  BiasedAttention           grouped-head causal attention with a log-distance bias per head and a position-dependent
+                            query temperature, no rotation
+  GatedDenseMLP             W_d (act(W_g h + b) * (W_u h + b)) + b
+  SharedSparseMLP           top-k experts of the plain form W_d act(W_u h), softmax over the chosen logits, plus a shared
+                            expert behind a per-token sigmoid gate
 
 Activations are fp32 tensors [rows, features]; matrices are stored in the serving dtype (bf16, or fp32 for the exact
 mode), vectors always in fp32.  A step's rows come with the metadata of utils/context.py: cu_seqlens_q, kv_lens (the
@@ -21,7 +31,7 @@ from __future__ import annotations
 import torch
 from torch import nn
 
-from nanovllm import ops
+from nanovllm import _C, ops
 from nanovllm.utils.context import get_context
 
 
@@ -37,7 +47,7 @@ class MergedRows(nn.Module):
     """Several projections of the same input stacked along their output features (one GEMM instead of several); a
     checkpoint's separate tensors land in their row ranges through `weight_loader(param, tensor, shard_name)`."""
 
-    def __init__(self, in_features: int, parts: dict[str, int], dtype=None):
+    def __init__(self, in_features: int, parts: dict[str, int], dtype=None, bias: bool = False):
         super().__init__()
         self.offsets, off = {}, 0
         for name, n in parts.items():
@@ -45,6 +55,10 @@ class MergedRows(nn.Module):
             off += n
         self.weight = nn.Parameter(torch.empty(off, in_features, dtype=dtype), requires_grad=False)
         self.weight.weight_loader = self._load
+        self.bias = None
+        if bias:  # fp32, zero where a part has none; loaded by row range like the weight
+            self.bias = _vector(off)
+            self.bias.weight_loader = self._load
 
     def _load(self, param, tensor, shard):
         off, n = self.offsets[shard]
@@ -56,6 +70,8 @@ class MergedRows(nn.Module):
         return y[:, off:off + n]
 
     def forward(self, x: torch.Tensor, exact: bool = False) -> torch.Tensor:
+        if self.bias is not None:
+            return ops.gemm_any_act(x, self.weight, bias=self.bias, exact=exact)
         return ops.gemm_any(x, self.weight, exact=exact)
 
 
@@ -159,3 +175,171 @@ class GroupedSparseMLP(nn.Module):
         act = ops.gemm_any_grouped(x, pair_token, self.gate, self.up, offsets, P, None, P)
         y = ops.gemm_any_grouped(act, None, self.down, None, offsets, P, pair_index, P)
         return ops.moe_combine_f32(y, x, ids, wts, self.E)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# pre-norm families with a depth-mixed residual stream
+# ---------------------------------------------------------------------------------------------------------------------
+_ACTS = {"silu": _C.ACT_SILU, "gelu_tanh": _C.ACT_GELU_TANH, "gelu": _C.ACT_GELU_ERF, "sigmoid": _C.ACT_SIGMOID, None: _C.ACT_NONE}
+CAUSAL = 2 ** 31 - 1   # "window" of plain causal attention
+
+
+class DepthMixedResidual:
+    """The residual stream of one step: slot 0 holds the embedding rows, slot i + 1 layer i's result
+    X_{i+1} = a + m f1(n1(a)) + m f2(n2(.)), where a - what layer i reads - is the weighted sum of the slots 0..i with the
+    previous layer's coefficients (layer 0 reads slot 0 itself).  The sum for layer i + 1 is written straight into slot
+    i + 2 and becomes X_{i+2} by the in-place residual updates.  One launch per layer boundary folds the last residual
+    update, the weighted sum and the next layer's first norm."""
+
+    def __init__(self, rows: int, width: int, n_layers: int, mult: float, eps: float, device, shift: float = 1.0):
+        self.stack = torch.empty((n_layers + 2, rows, width), dtype=torch.float32, device=device)  # slot 0: the caller's
+        self.n, self.mult, self.eps, self.shift = 1, mult, eps, shift
+        self._one = torch.ones(1, dtype=torch.float32, device=device)
+
+    @property
+    def current(self) -> torch.Tensor:
+        return self.stack[self.n]
+
+    def begin(self, norm_w: torch.Tensor) -> torch.Tensor:
+        """-> n(slot 0) for the first layer"""
+        return ops.depth_mix_f32(self.stack, 1, self._one, None, 0.0, norm_w, self.eps, self.shift)
+
+    def add_and_norm(self, y: torch.Tensor, norm_w: torch.Tensor | None):
+        """current += m * y; -> its norm (None without a weight)"""
+        return ops.add_rmsnorm_f32(self.current, y, self.mult, norm_w, self.eps, self.shift)
+
+    def next_layer(self, y: torch.Tensor | None, coef: torch.Tensor, norm_w: torch.Tensor | None):
+        """current += m * y (the layer's last sublayer); the weighted sum of all results so far opens the next slot;
+        -> its norm with the next layer's first norm weight (None after the last layer)"""
+        self.n += 1
+        return ops.depth_mix_f32(self.stack, self.n, coef, y, self.mult, norm_w, self.eps, self.shift)
+
+
+class MinGRUMixer(nn.Module):
+    """z = sigmoid(W_z h + b_z), u = W_x h + b_x, c = u + 1/2 (u >= 0) | sigmoid(u); S <- (1 - z) S + z c per channel;
+    out = W_o (S * silu(W_g h)).  The state [slots, width] is fp32."""
+
+    def __init__(self, width_in: int, width: int):
+        super().__init__()
+        self.n = width
+        self.zxg = MergedRows(width_in, {"z": width, "x": width, "g": width}, bias=True)
+        self.o = _matrix(width_in, width)
+        self.state = torch.tensor([])
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        ctx, off = get_context(), self.zxg.offsets
+        y = self.zxg(h)
+        s = ops.mingru_scan(y, off["z"][0], off["x"][0], off["g"][0], self.n, self.state, ctx.cu_seqlens_q, ctx.kv_lens,
+                            ctx.state_slots, ctx.max_seqlen_q)
+        return ops.gemm_any(s, self.o)
+
+
+class LatentAttention(nn.Module):
+    """[c | r] = W_dkv h; c <- rms(c) * w_c; k_h = [W_uk,h c | rot(r)], v_h = W_uv,h c; q_h = [q_h' | rot(q_h'')].
+    Cached per token: [c | rot(r)] only - ONE key/value row for all heads.  Scores and outputs are formed in the latent
+    space: q_h'.(W_uk,h c) = (W_uk,h^T q_h').c, sum_j p_j W_uv,h c_j = W_uv,h (sum_j p_j c_j), so the attention is
+    multi-query attention with key rows [c | r] of C + R channels whose first C channels are also the values; the two
+    per-head projections around it are batched GEMMs over head-major rows."""
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, rot_dims: int,
+                 rot_base: float, scale: float, eps: float):
+        super().__init__()
+        assert 0 <= rot_dims <= rot_dim and rot_dims % 2 == 0
+        self.H, self.D, self.R, self.Dv, self.C = heads, dim, rot_dim, vdim, kv_rank
+        self.rot_dims, self.rot_base, self.scale, self.eps = rot_dims, rot_base, scale, eps
+        self.qcg = MergedRows(width, {"q": heads * (dim + rot_dim), "dkv": kv_rank + rot_dim, "g": heads * vdim})
+        self.c_norm = _vector(kv_rank, 1.0)
+        self.uk_t = _matrix(heads, kv_rank, dim)   # W_uk,h transposed: the query-side projection into the latent space
+        self.uv = _matrix(heads, vdim, kv_rank)
+        self.uk_t.weight_loader = lambda p, t: p.data.copy_(t.view(heads, dim, kv_rank).transpose(1, 2))
+        self.uv.weight_loader = lambda p, t: p.data.copy_(t.view(heads, vdim, kv_rank))
+        self.o = _matrix(width, heads * vdim)
+        self.cache = torch.tensor([])
+
+    def cache_shape(self, num_blocks: int, block_size: int):
+        return (num_blocks, 1, block_size, self.C + self.R)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        ctx, m = get_context(), self.qcg
+        H, D, R, Dv, C = self.H, self.D, self.R, self.Dv, self.C
+        y = m(h)
+        qx = torch.empty((h.shape[0], H * (C + R)), dtype=torch.float32, device=h.device)
+        ops.latent_prepare(y, m.offsets["q"][0], m.offsets["dkv"][0], H, D, R, C, self.rot_dims, self.rot_base, self.c_norm,
+                           self.eps, ctx.cu_seqlens_q, ctx.kv_lens, self.cache, ctx.slot_mapping, qx)
+        ops.gemm_any_batched(m.cols(y, "q"), D + R, self.uk_t, qx, C + R)
+        o = ops.paged_attention_f32(qx, self.cache, self.cache, C + R, ctx.block_tables, ctx.cu_seqlens_q, ctx.kv_lens, H, 1,
+                                    C + R, C, ctx.block_size, CAUSAL, self.scale, _C.BIAS_NONE)
+        ov = torch.empty((h.shape[0], H * Dv), dtype=torch.float32, device=h.device)
+        ops.gemm_any_batched(o, C, self.uv, ov, Dv, gate=m.cols(y, "g"), gate_batch=Dv)
+        return ops.gemm_any(ov, self.o)
+
+
+class BiasedAttention(nn.Module):
+    """s_ij = scale * t(i) q_i . k_j - r1_h ln(1 + r2_h (i - j)), t(p) = 1 + coef ln(floor((p + 1) / every) + 1)
+    (every < 1: no temperature); causal, grouped key/value heads of separate key and value sizes, no rotation."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, temp_coef: float = 0.0,
+                 temp_every: int = 0):
+        super().__init__()
+        assert heads % kv_heads == 0
+        self.H, self.G, self.D, self.Dv, self.scale = heads, kv_heads, dim, vdim, scale
+        self.temp_coef, self.temp_every = temp_coef, temp_every
+        self.qkv = MergedRows(width, {"q": heads * dim, "k": kv_heads * dim, "v": kv_heads * vdim})
+        self.r1, self.r2 = _vector(heads), _vector(heads)
+        self.o = _matrix(width, heads * vdim)
+        self.k_cache = self.v_cache = torch.tensor([])
+
+    def cache_shapes(self, num_blocks: int, block_size: int):
+        return (num_blocks, self.G, block_size, self.D), (num_blocks, self.G, block_size, self.Dv)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        ctx, m = get_context(), self.qkv
+        y = m(h)
+        ops.kv_store_temp(y, m.offsets["q"][0], m.offsets["k"][0], m.offsets["v"][0], self.temp_coef, self.temp_every,
+                          ctx.cu_seqlens_q, ctx.kv_lens, self.k_cache, self.v_cache, ctx.slot_mapping, self.H, self.G,
+                          self.D, self.Dv, ctx.block_size)
+        o = ops.paged_attention_f32(m.cols(y, "q"), self.k_cache, self.v_cache, self.Dv, ctx.block_tables, ctx.cu_seqlens_q,
+                                    ctx.kv_lens, self.H, self.G, self.D, self.Dv, ctx.block_size, CAUSAL, self.scale,
+                                    _C.BIAS_LOG, self.r1, self.r2)
+        return ops.gemm_any(o, self.o)
+
+
+class GatedDenseMLP(nn.Module):
+    def __init__(self, width: int, ff: int, act: str = "gelu_tanh"):
+        super().__init__()
+        self.act = _ACTS[act]
+        self.gate, self.up, self.down = _matrix(ff, width), _matrix(ff, width), _matrix(width, ff)
+        self.gate_b, self.up_b, self.down_b = _vector(ff), _vector(ff), _vector(width)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        a = ops.gemm_any_act(h, self.gate, bias=self.gate_b, act=self.act, w2=self.up, bias2=self.up_b)
+        return ops.gemm_any_act(a, self.down, bias=self.down_b)
+
+
+class SharedSparseMLP(nn.Module):
+    """Router logits in true 32-bit; the `top_k` largest, weights = softmax over them; experts W_d act(W_u h) without
+    biases; shared_ff > 0: a shared expert of the same form for every token, times sigmoid(w_sg . h) - that gate's row
+    rides behind the router's rows in one projection."""
+
+    def __init__(self, width: int, ff: int, experts: int, top_k: int, shared_ff: int = 0, act: str = "gelu"):
+        super().__init__()
+        assert 1 <= top_k <= experts
+        self.E, self.top_k, self.act, self.shared = experts, top_k, _ACTS[act], shared_ff > 0
+        self.router = MergedRows(width, {"router": experts, "sg": 1} if self.shared else {"router": experts})
+        self.up, self.down = _matrix(experts, ff, width), _matrix(experts, width, ff)
+        for p in (self.up, self.down):
+            p.weight_loader = lambda param, tensor, expert: param.data[expert].copy_(tensor)
+        if self.shared:
+            self.shared_up, self.shared_down = _matrix(shared_ff, width), _matrix(width, shared_ff)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        z = self.router(h, exact=True)
+        ids, wts = ops.route_topk(z, self.E, self.top_k)
+        offsets, pair_token, pair_index = ops.moe_sort(ids, self.E)
+        P = ids.numel()
+        a = ops.gemm_any_grouped_act(h, pair_token, self.up, None, self.act, offsets, P, None, P)
+        y = ops.gemm_any_grouped_act(a, None, self.down, None, _C.ACT_NONE, offsets, P, pair_index, P)
+        if not self.shared:
+            return ops.moe_combine_shared(y, ids, wts, h.shape[1])
+        sh = ops.gemm_any(ops.gemm_any_act(h, self.shared_up, act=self.act), self.shared_down)
+        return ops.moe_combine_shared(y, ids, wts, h.shape[1], sh, z[:, self.E:])

@@ -6,6 +6,7 @@ from nanovllm.models.gazutar import GazutarConfig, GazutarForCausalLM
 from nanovllm.models.llama import LlamaForCausalLM
 from nanovllm.models.qwen3 import Qwen3ForCausalLM
 from nanovllm.models.qwen3_moe import Qwen3MoeForCausalLM
+from nanovllm.models.zedirax import ZediraxConfig, ZediraxForCausalLM
 
 model_dict = {
     "Qwen3ForCausalLM": Qwen3ForCausalLM,
@@ -13,11 +14,13 @@ model_dict = {
     "LlamaForCausalLM": LlamaForCausalLM,
     "Qwen3MoeForCausalLM": Qwen3MoeForCausalLM,
     "Gazutar": GazutarForCausalLM,
+    "Zedirax": ZediraxForCausalLM,
 }
 
 # designs whose config.json is not a transformers configuration: {"architecture": <name>, ...} -> the reader of it
 native_configs = {
     "Gazutar": GazutarConfig,
+    "Zedirax": ZediraxConfig,
 }
 
 

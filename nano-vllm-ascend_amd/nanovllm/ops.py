@@ -985,10 +985,12 @@ def gemm_any_grouped(x, x_rows, w, w2, group_offsets, rows_max: int, y_rows, y_r
     return y
 
 
-def embedding_f32(ids, table) -> torch.Tensor:
+def embedding_f32(ids, table, out=None) -> torch.Tensor:
     require_gpu(ids, table)
     assert ids.dtype == torch.int64 and ids.is_contiguous() and table.is_contiguous()
-    out = torch.empty((ids.numel(), table.shape[1]), dtype=_F32, device=table.device)
+    if out is None:
+        out = torch.empty((ids.numel(), table.shape[1]), dtype=_F32, device=table.device)
+    assert out.shape == (ids.numel(), table.shape[1]) and out.dtype == _F32 and out.is_contiguous()
     check(lib.mi_embedding_f32(ptr(ids), ptr(table), _dt(table), ptr(out), ids.numel(), table.shape[1], table.shape[0],
                                stream()), "mi_embedding_f32")
     return out
@@ -1118,4 +1120,179 @@ def moe_combine_f32(y, h, ids, wts, n_experts: int) -> torch.Tensor:
     out = torch.empty((T, width), dtype=_F32, device=h.device)
     check(lib.mi_moe_combine_f32(ptr(y), ptr(h), h.stride(0), ptr(ids), ptr(wts), T, top_k, n_experts, width, ptr(out),
                                  width, stream()), "mi_moe_combine_f32")
+    return out
+
+
+# ---- pre-norm 32-bit families: epilogue / batched projections, residual stack, minimal gated recurrence, latent and
+# log-distance-biased attention, plain top-k routing (csrc/gemm_any.hip, csrc/seqmix.hip)
+def gemm_any_act(x, w, bias=None, act: int = _C.ACT_NONE, w2=None, bias2=None, alpha: float = 1.0, exact: bool = False,
+                 out=None) -> torch.Tensor:
+    """alpha * act(x w^T + bias), or with w2: alpha * act(x w^T + bias) * (x w2^T + bias2)."""
+    require_gpu(x, w)
+    _f32(x, out, bias, bias2)
+    assert x.dim() == 2 and w.dim() == 2 and w.is_contiguous() and x.shape[1] == w.shape[1], (x.shape, w.shape)
+    assert w2 is None or (w2.shape == w.shape and w2.dtype == w.dtype and w2.is_contiguous())
+    M, K = x.shape
+    N = w.shape[0]
+    assert (bias is None or bias.numel() == N) and (bias2 is None or (bias2.numel() == N and w2 is not None))
+    if out is None:
+        out = torch.empty((M, N), dtype=_F32, device=x.device)
+    assert out.shape == (M, N)
+    check(lib.mi_gemm_any_act(ptr(x), x.stride(0) if M > 1 else K, ptr(w), ptr(w2), _dt(w), ptr(bias), ptr(bias2), int(act),
+                              ptr(out), out.stride(0) if M > 1 else N, M, N, K, float(alpha), int(exact), stream()),
+          "mi_gemm_any_act")
+    return out
+
+
+def gemm_any_grouped_act(x, x_rows, w, w2, act: int, group_offsets, rows_max: int, y_rows, y_rows_total: int,
+                         exact: bool = False):
+    """gemm_any_grouped with the activation named: per group y = act(x w[g]^T) (* (x w2[g]^T) with w2)."""
+    require_gpu(x, w, group_offsets)
+    _f32(x)
+    _i32(x_rows, y_rows, group_offsets)
+    assert w.dim() == 3 and w.is_contiguous() and (w2 is None or (w2.shape == w.shape and w2.is_contiguous() and w2.dtype == w.dtype))
+    G, N, K = w.shape
+    assert x.shape[1] == K and group_offsets.numel() >= G + 1
+    y = torch.empty((y_rows_total, N), dtype=_F32, device=x.device)
+    check(lib.mi_gemm_any_grouped_act(ptr(x), x.stride(0), ptr(x_rows), ptr(w), ptr(w2), _dt(w), int(act), ptr(group_offsets),
+                                      G, rows_max, ptr(y), N, ptr(y_rows), N, K, int(exact), stream()),
+          "mi_gemm_any_grouped_act")
+    return y
+
+
+def gemm_any_batched(x, x_batch: int, w, out, out_batch: int, gate=None, gate_batch: int = 0, exact: bool = False):
+    """Per batch b (a head): out[:, b*out_batch : +N] = x[:, b*x_batch : +K] @ w[b].T (* sigmoid(gate[:, b*gate_batch : +N]));
+    x, out, gate: [rows, >= n_batch * stride] fp32 with unit inner stride."""
+    require_gpu(x, w, out)
+    _f32(x, out, gate)
+    B, N, K = w.shape
+    M = x.shape[0]
+    assert w.is_contiguous() and out.shape[0] == M and (gate is None or gate.shape[0] == M)
+    assert (B - 1) * x_batch + K <= x.shape[1] and (B - 1) * out_batch + N <= out.shape[1]
+    assert gate is None or (B - 1) * gate_batch + N <= gate.shape[1]
+    check(lib.mi_gemm_any_batched(ptr(x), x.stride(0), x_batch, ptr(w), _dt(w), ptr(out), out.stride(0), out_batch, ptr(gate),
+                                  gate.stride(0) if gate is not None else 0, gate_batch, B, M, N, K, int(exact), stream()),
+          "mi_gemm_any_batched")
+    return out
+
+
+def paged_attention_f32(q, k_cache, v_cache, ldv: int, block_tables, cu_q, kv_lens, H: int, G: int, D: int, Dv: int,
+                        block_size: int, window: int, scale: float, bias_kind: int = _C.BIAS_NONE, bias_p1=None, bias_p2=None,
+                        gate=None) -> torch.Tensor:
+    """Paged causal attention over fp32 queries; see mi_paged_attention_f32 (bias kinds, values inside the key rows)."""
+    require_gpu(q, k_cache, v_cache, block_tables, cu_q, kv_lens)
+    _f32(q, gate, bias_p1, bias_p2)
+    _i32(block_tables, cu_q, kv_lens)
+    rows, n_seqs = q.shape[0], kv_lens.numel()
+    assert q.shape[1] >= H * D and cu_q.numel() == n_seqs + 1 and block_tables.shape[0] >= n_seqs
+    assert k_cache.dtype == v_cache.dtype
+    assert bias_kind != _C.BIAS_LOG or (bias_p1.numel() == H and bias_p2.numel() == H)
+    out = torch.empty((rows, H * Dv), dtype=_F32, device=q.device)
+    check(lib.mi_paged_attention_f32(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), int(ldv), _dt(k_cache),
+                                     ptr(block_tables), block_tables.shape[1], ptr(cu_q), ptr(kv_lens), n_seqs, rows, H, G,
+                                     D, Dv, block_size, int(min(window, 2 ** 31 - 1)), float(scale), int(bias_kind),
+                                     ptr(bias_p1), ptr(bias_p2), ptr(gate), gate.stride(0) if gate is not None else 0,
+                                     ptr(out), out.stride(0), stream()), "mi_paged_attention_f32")
+    return out
+
+
+def add_rmsnorm_f32(res, y, mult: float, w, eps: float, shift: float = 0.0, out=None):
+    """res += mult * y in place (y None: unchanged); w given: returns res / rms(res) * (w + shift), else None."""
+    require_gpu(res)
+    _f32(res, y, w, out)
+    rows, width = res.shape
+    assert y is None or y.shape == res.shape
+    if w is not None:
+        assert w.numel() == width
+        if out is None:
+            out = torch.empty((rows, width), dtype=_F32, device=res.device)
+    check(lib.mi_add_rmsnorm_f32(ptr(res), res.stride(0), ptr(y), y.stride(0) if y is not None else 0, float(mult), ptr(w),
+                                 float(shift), float(eps), ptr(out), out.stride(0) if out is not None else 0, rows, width,
+                                 stream()), "mi_add_rmsnorm_f32")
+    return out
+
+
+def depth_mix_f32(stack, n: int, coef, y, mult: float, norm_w, eps: float, shift: float = 0.0):
+    """stack [slots, rows, width]: slot n-1 += mult * y (y None: unchanged); slot n = sum_{j<n} coef[j] * slot j; returns
+    slot n normed with (norm_w + shift), or None without norm_w."""
+    require_gpu(stack, coef)
+    _f32(stack, coef, y, norm_w)
+    slots, rows, width = stack.shape
+    assert stack.is_contiguous() and 1 <= n < slots and coef.numel() == n
+    h = torch.empty((rows, width), dtype=_F32, device=stack.device) if norm_w is not None else None
+    check(lib.mi_depth_mix_f32(ptr(stack), rows * width, n, ptr(coef), ptr(y), y.stride(0) if y is not None else 0,
+                               float(mult), ptr(norm_w), float(shift), float(eps), ptr(h), width, rows, width, stream()),
+          "mi_depth_mix_f32")
+    return h
+
+
+def mingru_scan(proj, z_off: int, x_off: int, g_off: int, width: int, state, cu_q, kv_lens, slot_ids,
+                max_rows_per_seq: int) -> torch.Tensor:
+    require_gpu(proj, state)
+    _f32(proj, state)
+    _i32(cu_q, kv_lens, slot_ids)
+    rows, n_seqs = proj.shape[0], kv_lens.numel()
+    assert state.is_contiguous() and state.shape[1] == width and max(z_off, x_off, g_off) + width <= proj.shape[1]
+    out = torch.empty((rows, width), dtype=_F32, device=proj.device)
+    ws = None
+    if max_rows_per_seq > 64:
+        ws = torch.empty(lib.mi_mingru_scan_workspace_elems(rows, n_seqs, width), dtype=_F32, device=proj.device)
+    check(lib.mi_mingru_scan(ptr(proj), proj.stride(0), z_off, x_off, g_off, ptr(state), ptr(cu_q), ptr(kv_lens),
+                             ptr(slot_ids), n_seqs, rows, int(max_rows_per_seq), width, ptr(ws), ptr(out), width, stream()),
+          "mi_mingru_scan")
+    return out
+
+
+def kv_store_temp(proj, q_off: int, k_off: int, v_off: int, temp_coef: float, temp_every: int, cu_q, kv_lens, k_cache,
+                  v_cache, slots, H: int, G: int, D: int, Dv: int, block_size: int) -> None:
+    require_gpu(proj, k_cache, v_cache, slots)
+    _f32(proj)
+    _i32(slots, cu_q, kv_lens)
+    rows = proj.shape[0]
+    assert slots.numel() == rows and k_cache.dtype == v_cache.dtype
+    assert k_cache.shape[1:] == (G, block_size, D) and v_cache.shape[1:] == (G, block_size, Dv), (k_cache.shape, v_cache.shape)
+    assert max(q_off + H * D, k_off + G * D, v_off + G * Dv) <= proj.shape[1]
+    check(lib.mi_kv_store_temp(ptr(proj), proj.stride(0), q_off, k_off, v_off, float(temp_coef), int(temp_every), ptr(cu_q),
+                               ptr(kv_lens), kv_lens.numel(), ptr(k_cache), ptr(v_cache), _dt(k_cache), ptr(slots), rows, H,
+                               G, D, Dv, block_size, stream()), "mi_kv_store_temp")
+
+
+def latent_prepare(proj, q_off: int, c_off: int, H: int, D: int, R: int, C: int, rot_dims: int, rot_base: float, norm_w,
+                   eps: float, cu_q, kv_lens, cache, slots, qx) -> None:
+    require_gpu(proj, cache, slots, qx)
+    _f32(proj, norm_w, qx)
+    _i32(slots, cu_q, kv_lens)
+    rows = proj.shape[0]
+    assert slots.numel() == rows and norm_w.numel() == C and cache.shape[-1] == C + R and cache.is_contiguous()
+    assert qx.shape == (rows, H * (C + R)) and max(q_off + H * (D + R), c_off + C + R) <= proj.shape[1]
+    check(lib.mi_latent_prepare(ptr(proj), proj.stride(0), q_off, c_off, H, D, R, C, int(rot_dims), float(rot_base),
+                                ptr(norm_w), float(eps), ptr(cu_q), ptr(kv_lens), kv_lens.numel(), ptr(cache), _dt(cache),
+                                ptr(slots), ptr(qx), qx.stride(0), rows, stream()), "mi_latent_prepare")
+
+
+def route_topk(logits, n_outputs: int, top_k: int):
+    """The top_k largest of the first n_outputs columns; weights = softmax over the chosen logits."""
+    require_gpu(logits)
+    _f32(logits)
+    T = logits.shape[0]
+    assert n_outputs <= logits.shape[1]
+    ids = torch.empty((T, top_k), dtype=torch.int32, device=logits.device)
+    wts = torch.empty((T, top_k), dtype=_F32, device=logits.device)
+    check(lib.mi_route_topk(ptr(logits), logits.stride(0), T, n_outputs, top_k, ptr(ids), ptr(wts), stream()),
+          "mi_route_topk")
+    return ids, wts
+
+
+def moe_combine_shared(y, ids, wts, width: int, shared=None, shared_gate=None) -> torch.Tensor:
+    """sum_k wts[t][k] * y[t * top_k + k] (+ sigmoid(shared_gate[t]) * shared[t])."""
+    require_gpu(y, ids, wts)
+    _f32(y, wts, shared)
+    T, top_k = ids.shape
+    assert y.shape == (T * top_k, width) and y.is_contiguous()
+    assert shared is None or (shared.shape == (T, width) and shared_gate is not None and shared_gate.dtype == _F32)
+    out = torch.empty((T, width), dtype=_F32, device=y.device)
+    check(lib.mi_moe_combine_shared(ptr(y), ptr(ids), ptr(wts), T, top_k, width, ptr(shared),
+                                    shared.stride(0) if shared is not None else 0, ptr(shared_gate),
+                                    shared_gate.stride(0) if shared_gate is not None else 0, ptr(out), width, stream()),
+          "mi_moe_combine_shared")
     return out
