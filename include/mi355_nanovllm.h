@@ -767,9 +767,10 @@ int mi_kv_store_temp(float* proj, int64_t ld, int q_off, int k_off, int v_off, f
                      const int32_t* slots, int rows, int H, int G, int D, int Dv, int block_size, mi_stream stream);
 /* Latent attention, per row: cache row [slot] = [rms(c) * norm_w | rot(r)] (c: C entries at c_off, r: the R behind
  * them); qx[row][h][C .. C + R) = rot(q_h[D .. D + R)) for every head (q heads of D + R entries at q_off).  rot turns
- * the first rot_dims entries: pairs (i, i + rot_dims/2), angle pos * rot_base^(-2 i / rot_dims). */
+ * the first rot_dims entries: pairs (i, i + rot_dims/2), angle pos * inv_freq[i] (a table of rot_dims/2 floats:
+ * base^(-2 i / rot_dims)). */
 int mi_latent_prepare(const float* proj, int64_t ld, int q_off, int c_off, int H, int D, int R, int C, int rot_dims,
-                      float rot_base, const float* norm_w, float eps, const int32_t* cu_q, const int32_t* kv_lens,
+                      const float* inv_freq, const float* norm_w, float eps, const int32_t* cu_q, const int32_t* kv_lens,
                       int n_seqs, void* cache, int cache_dtype, const int32_t* slots, float* qx, int64_t ldqx, int rows,
                       mi_stream stream);
 /* ids = the top_k largest logits (descending; equal: lower index), weights = softmax over those.  n_outputs <= 512. */

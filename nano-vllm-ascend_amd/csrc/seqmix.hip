@@ -1109,10 +1109,12 @@ __global__ __launch_bounds__(256) void kv_store_temp_kernel(float* __restrict__ 
 // whole row, values = its first C channels.  The rotated part of every query head (R entries at q_off + h * (D + R) + D)
 // is rotated and written to qx[row][h][C ..] - the head's absorbed key-space query [W_uk^T q | rot(q_r)] whose first C
 // entries a batched projection fills in.  Rotation: the first `dims` entries, pairs (i, i + dims / 2), angle
-// pos * base^(-2 i / dims), computed in fp32 (powf / sincosf of the device library).
+// pos * inv_freq[i] formed and turned into sine and cosine in fp32 (sincosf of the device library); inv_freq [dims / 2]
+// is the host's table of base^(-2 i / dims), rounded once from double.
 template <typename TC>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __restrict__ proj, int64_t ld, int q_off,
-                                                             int c_off, int H, int D, int R, int C, int dims, float base,
+                                                             int c_off, int H, int D, int R, int C, int dims,
+                                                             const float* __restrict__ inv_freq,
                                                              const float* __restrict__ norm_w, float eps,
                                                              const int32_t* __restrict__ cu_q,
                                                              const int32_t* __restrict__ kv_lens, int n_seqs,
@@ -1138,7 +1140,7 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(const float* __rest
     float v = src[e];
     if (e < dims) {
       const int f = e < half ? e : e - half;
-      const float ang = (float)pos * powf(base, -2.f * (float)f / (float)dims);
+      const float ang = (float)pos * inv_freq[f];
       float sn, cs;
       sincosf(ang, &sn, &cs);
       v = e < half ? src[e] * cs - src[e + half] * sn : src[e] * cs + src[e - half] * sn;
@@ -1508,20 +1510,21 @@ extern "C" int mi_kv_store_temp(float* proj, int64_t ld, int q_off, int k_off, i
 }
 
 extern "C" int mi_latent_prepare(const float* proj, int64_t ld, int q_off, int c_off, int H, int D, int R, int C,
-                                 int rot_dims, float rot_base, const float* norm_w, float eps, const int32_t* cu_q,
+                                 int rot_dims, const float* inv_freq, const float* norm_w, float eps, const int32_t* cu_q,
                                  const int32_t* kv_lens, int n_seqs, void* cache, int cache_dtype, const int32_t* slots,
                                  float* qx, int64_t ldqx, int rows, mi_stream stream) {
   if (!proj || !norm_w || !cu_q || !kv_lens || !cache || !slots || !qx || rows < 0 || n_seqs < 1) return MI_EINVAL;
   if (H < 1 || D < 0 || R < 0 || C < 1 || rot_dims < 0 || rot_dims > R || rot_dims % 2 || ldqx < (int64_t)H * (C + R))
     return MI_EINVAL;
+  if (rot_dims > 0 && !inv_freq) return MI_EINVAL;
   if (rows == 0) return MI_OK;
   if (cache_dtype == MI_DTYPE_BF16)
     hipLaunchKernelGGL((latent_prepare_kernel<uint16_t>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, c_off, H, D,
-                       R, C, rot_dims, rot_base, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<uint16_t*>(cache), slots,
+                       R, C, rot_dims, inv_freq, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<uint16_t*>(cache), slots,
                        qx, ldqx);
   else if (cache_dtype == MI_DTYPE_F32)
     hipLaunchKernelGGL((latent_prepare_kernel<float>), dim3(rows), dim3(256), 0, S(stream), proj, ld, q_off, c_off, H, D, R,
-                       C, rot_dims, rot_base, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<float*>(cache), slots, qx,
+                       C, rot_dims, inv_freq, norm_w, eps, cu_q, kv_lens, n_seqs, static_cast<float*>(cache), slots, qx,
                        ldqx);
   else return MI_EINVAL;
   return check_launch();

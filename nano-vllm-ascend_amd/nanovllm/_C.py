@@ -199,7 +199,7 @@ _SIGNATURES = {
                                c_int64, _p]),
     "mi_kv_store_temp": (c_int, [_p, c_int64, c_int, c_int, c_int, c_float, c_int, _p, _p, c_int, _p, _p, c_int, _p, c_int,
                                  c_int, c_int, c_int, c_int, c_int, _p]),
-    "mi_latent_prepare": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _p, c_float, _p,
+    "mi_latent_prepare": (c_int, [_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _p, _p, c_float, _p,
                                   _p, c_int, _p, c_int, _p, _p, c_int64, c_int, _p]),
     "mi_route_topk": (c_int, [_p, c_int64, c_int, c_int, c_int, _p, _p, _p]),
     "mi_moe_combine_shared": (c_int, [_p, _p, _p, c_int, c_int, c_int, _p, c_int64, _p, c_int64, _p, c_int64, _p]),

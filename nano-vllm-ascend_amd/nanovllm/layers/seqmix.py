@@ -184,6 +184,11 @@ _ACTS = {"silu": _C.ACT_SILU, "gelu_tanh": _C.ACT_GELU_TANH, "gelu": _C.ACT_GELU
 CAUSAL = 2 ** 31 - 1   # "window" of plain causal attention
 
 
+def rotary_inv_freq(dims: int, base: float) -> torch.Tensor:
+    f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)] or [0.0]
+    return torch.tensor(f, dtype=torch.float64).to(torch.float32)
+
+
 class DepthMixedResidual:
     """The residual stream of one step: slot 0 holds the embedding rows, slot i + 1 layer i's result
     X_{i+1} = a + m f1(n1(a)) + m f2(n2(.)), where a - what layer i reads - is the weighted sum of the slots 0..i with the
@@ -191,10 +196,11 @@ class DepthMixedResidual:
     i + 2 and becomes X_{i+2} by the in-place residual updates.  One launch per layer boundary folds the last residual
     update, the weighted sum and the next layer's first norm."""
 
-    def __init__(self, rows: int, width: int, n_layers: int, mult: float, eps: float, device, shift: float = 1.0):
-        self.stack = torch.empty((n_layers + 2, rows, width), dtype=torch.float32, device=device)  # slot 0: the caller's
+    def __init__(self, rows: int, width: int, n_layers: int, mult: float, eps: float, unit: torch.Tensor, shift: float = 1.0):
+        """unit: a device tensor holding 1.0 (the first layer's only coefficient)"""
+        self.stack = torch.empty((n_layers + 2, rows, width), dtype=torch.float32, device=unit.device)  # slot 0: the caller's
         self.n, self.mult, self.eps, self.shift = 1, mult, eps, shift
-        self._one = torch.ones(1, dtype=torch.float32, device=device)
+        self._one = unit
 
     @property
     def current(self) -> torch.Tensor:
@@ -247,6 +253,8 @@ class LatentAttention(nn.Module):
         assert 0 <= rot_dims <= rot_dim and rot_dims % 2 == 0
         self.H, self.D, self.R, self.Dv, self.C = heads, dim, rot_dim, vdim, kv_rank
         self.rot_dims, self.rot_base, self.scale, self.eps = rot_dims, rot_base, scale, eps
+        # base^(-2 i / dims) in double, rounded once (a buffer, not a checkpoint tensor)
+        self.register_buffer("inv_freq", rotary_inv_freq(rot_dims, rot_base), persistent=False)
         self.qcg = MergedRows(width, {"q": heads * (dim + rot_dim), "dkv": kv_rank + rot_dim, "g": heads * vdim})
         self.c_norm = _vector(kv_rank, 1.0)
         self.uk_t = _matrix(heads, kv_rank, dim)   # W_uk,h transposed: the query-side projection into the latent space
@@ -264,7 +272,7 @@ class LatentAttention(nn.Module):
         H, D, R, Dv, C = self.H, self.D, self.R, self.Dv, self.C
         y = m(h)
         qx = torch.empty((h.shape[0], H * (C + R)), dtype=torch.float32, device=h.device)
-        ops.latent_prepare(y, m.offsets["q"][0], m.offsets["dkv"][0], H, D, R, C, self.rot_dims, self.rot_base, self.c_norm,
+        ops.latent_prepare(y, m.offsets["q"][0], m.offsets["dkv"][0], H, D, R, C, self.rot_dims, self.inv_freq, self.c_norm,
                            self.eps, ctx.cu_seqlens_q, ctx.kv_lens, self.cache, ctx.slot_mapping, qx)
         ops.gemm_any_batched(m.cols(y, "q"), D + R, self.uk_t, qx, C + R)
         o = ops.paged_attention_f32(qx, self.cache, self.cache, C + R, ctx.block_tables, ctx.cu_seqlens_q, ctx.kv_lens, H, 1,

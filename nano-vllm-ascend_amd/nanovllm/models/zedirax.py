@@ -95,6 +95,7 @@ class ZediraxForCausalLM(nn.Module):
         self.embed = nn.Parameter(torch.empty(V, W), requires_grad=False)
         self.layers = nn.ModuleList([ZediraxLayer(config, i) for i in range(len(config.layers))])
         self.final_norm = _vector(W)
+        self.register_buffer("unit", torch.ones(1, dtype=torch.float32), persistent=False)
         self.head = nn.Parameter(torch.empty(V, W), requires_grad=False)
         self.trace_layers: list | None = None  # bring-up hook: receives a copy of what every layer hands on
 
@@ -230,7 +231,7 @@ class ZediraxForCausalLM(nn.Module):
     # ---- one step over the rows the context describes ----------------------------------------------------------------
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor | None = None) -> torch.Tensor:
         cfg, n = self.config, len(self.layers)
-        res = DepthMixedResidual(input_ids.numel(), cfg.hidden_size, n, cfg.residual_mult, cfg.norm_eps, self.embed.device)
+        res = DepthMixedResidual(input_ids.numel(), cfg.hidden_size, n, cfg.residual_mult, cfg.norm_eps, self.unit)
         ops.embedding_f32(input_ids, self.embed, out=res.stack[0])
         h = res.begin(self.layers[0].norm1)
         for i, layer in enumerate(self.layers):

@@ -1257,15 +1257,16 @@ def kv_store_temp(proj, q_off: int, k_off: int, v_off: int, temp_coef: float, te
                                G, D, Dv, block_size, stream()), "mi_kv_store_temp")
 
 
-def latent_prepare(proj, q_off: int, c_off: int, H: int, D: int, R: int, C: int, rot_dims: int, rot_base: float, norm_w,
+def latent_prepare(proj, q_off: int, c_off: int, H: int, D: int, R: int, C: int, rot_dims: int, inv_freq, norm_w,
                    eps: float, cu_q, kv_lens, cache, slots, qx) -> None:
     require_gpu(proj, cache, slots, qx)
-    _f32(proj, norm_w, qx)
+    _f32(proj, norm_w, qx, inv_freq)
     _i32(slots, cu_q, kv_lens)
     rows = proj.shape[0]
+    assert inv_freq.is_cuda and inv_freq.numel() >= rot_dims // 2
     assert slots.numel() == rows and norm_w.numel() == C and cache.shape[-1] == C + R and cache.is_contiguous()
     assert qx.shape == (rows, H * (C + R)) and max(q_off + H * (D + R), c_off + C + R) <= proj.shape[1]
-    check(lib.mi_latent_prepare(ptr(proj), proj.stride(0), q_off, c_off, H, D, R, C, int(rot_dims), float(rot_base),
+    check(lib.mi_latent_prepare(ptr(proj), proj.stride(0), q_off, c_off, H, D, R, C, int(rot_dims), ptr(inv_freq),
                                 ptr(norm_w), float(eps), ptr(cu_q), ptr(kv_lens), kv_lens.numel(), ptr(cache), _dt(cache),
                                 ptr(slots), ptr(qx), qx.stride(0), rows, stream()), "mi_latent_prepare")
 
