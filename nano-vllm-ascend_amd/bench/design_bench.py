@@ -1,5 +1,5 @@
 """Prefill and decode throughput of a model design beside the framework's closest existing model at equal size
-(`python bench.py --design gazutar`): random weights, layer sizes that resemble a real model's, both models through the same
+(`python bench.py --design gazutar | zedirax`): random weights, layer sizes that resemble a real model's, both models through the same
 engine entry points (add_request / step), each served the way the framework serves it (Qwen3-MoE: captured prefill and
 decode steps; Gazutar: what ModelRunner reports in `served_as`).
 
@@ -32,6 +32,44 @@ def gazutar_config(s: dict) -> dict:
     layers = [dict(rec if i % 2 == 0 else att, mlp=ff) for i in range(s["layers"])]
     return {"architecture": "Gazutar", "vocab": s["vocab"], "width": s["width"], "logit_scale": 1.0, "norm": {"eps": 1e-6},
             "layers": layers}
+
+
+def zedirax_config(s: dict) -> dict:
+    """Recurrence / biased attention / recurrence / latent attention, sparse feed-forwards with a shared expert of one
+    expert's size (the third layer: a dense gated one of two model widths).  The latent attention caches 192 + 64 channels
+    per token for all heads."""
+    W, D = s["width"], s["dim"]
+    rec = {"type": "mingru", "mixer": {"width": W}}
+    att = {"type": "attention", "mixer": {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": D, "vdim": D, "scale": D ** -0.5,
+                                          "q_temp": {"coef": 0.1, "every": 512}}}
+    lat = {"type": "latent_attention", "mixer": {"heads": s["heads"], "dim": D, "rot_dim": 64, "vdim": D, "kv_rank": 192,
+                                                 "scale": (D + 64) ** -0.5, "rot": {"base": 10000.0, "dims": 64}}}
+    moe = {"kind": "moe", "expert": {"ff": s["ff"]}, "router": {"experts": s["experts"], "top": s["top"]}, "shared": {"ff": s["ff"]}}
+    dense = {"kind": "dense", "ff": 2 * W}
+    order = [(rec, moe), (att, moe), (rec, dense), (lat, moe)]
+    layers = [dict(order[i % 4][0], mlp=order[i % 4][1]) for i in range(s["layers"])]
+    return {"architecture": "Zedirax", "vocab": s["vocab"], "width": W, "residual_mult": 0.7, "norm": {"eps": 1e-6}, "layers": layers}
+
+
+def zedirax_decode_weight_bytes(cfg: dict, batch: int) -> float:
+    """bf16 weight bytes one decode step of `batch` rows streams (every projection, the experts the rows can reach, head)."""
+    W, n = cfg["width"], 0
+    for l in cfg["layers"]:
+        m = l["mixer"]
+        if l["type"] == "mingru":
+            n += 4 * W * m["width"]
+        elif l["type"] == "attention":
+            n += W * (m["heads"] * m["dim"] + m["kv_heads"] * (m["dim"] + m["vdim"])) + m["heads"] * m["vdim"] * W
+        else:
+            H, D, R, Dv, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            n += W * (H * (D + R) + C + R + H * Dv) + H * C * (D + Dv) + H * Dv * W
+        ml = l["mlp"]
+        if ml["kind"] == "dense":
+            n += 3 * W * ml["ff"]
+        else:
+            hit = min(ml["router"]["experts"], batch * ml["router"]["top"])
+            n += hit * 2 * W * ml["expert"]["ff"] + (ml["router"]["experts"] + 1) * W + 2 * W * ml["shared"]["ff"]
+    return 2.0 * (n + cfg["vocab"] * W)
 
 
 def qwen3_moe_config(s: dict) -> dict:
@@ -106,6 +144,9 @@ def run_model(cfg: dict, batch: int, prompt_len: int, steps: int, warmup: int, *
 
 def main(args) -> dict:
     batch, prompt_len = 32, 1024
+    design = getattr(args, "design", None) or "gazutar"
+    if design == "zedirax":
+        return main_zedirax(args, batch, prompt_len)
     out = {"metric": "design_throughput", "design": "gazutar", "closest_model": "Qwen3MoeForCausalLM", "unit": "tokens/s",
            "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
            "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
@@ -125,6 +166,36 @@ def main(args) -> dict:
             entry[label] = r
         if "gazutar" in entry and "qwen3_moe" in entry:
             entry["gazutar_vs_qwen3_moe"] = {k: entry["gazutar"][k] / entry["qwen3_moe"][k] for k in ("prefill_tok_s", "decode_tok_s")}
+        out["sizes"][name] = entry
+    print(json.dumps(out), flush=True)
+    return out
+
+
+def main_zedirax(args, batch: int, prompt_len: int) -> dict:
+    """Zedirax beside Gazutar - the closest existing model: the same row-step engine path, fp32 residual, pages plus state
+    slots, alternating recurrent and attention mixers, sparse feed-forwards - at equal width, depth, heads, experts and
+    vocabulary; Qwen3-MoE at that size rides along (`--design-models` picks)."""
+    out = {"metric": "design_throughput", "design": "zedirax", "closest_model": "Gazutar", "unit": "tokens/s",
+           "dtype": "bf16", "data": "synthetic (random weights, random prompts)", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "batch": batch, "prompt_len": prompt_len, "sizes": {}}
+    only_sizes = [x for x in getattr(args, "design_sizes", "").split(",") if x]
+    only_models = [x for x in getattr(args, "design_models", "").split(",") if x] or ["zedirax", "gazutar"]
+    for name, s in SIZES.items():
+        if only_sizes and name not in only_sizes:
+            continue
+        entry = {"shape": s}
+        zc = zedirax_config(s)
+        for label, cfg, wb in (("zedirax", zc, zedirax_decode_weight_bytes(zc, batch)),
+                               ("gazutar", gazutar_config(s), decode_weight_bytes(s, batch, True)),
+                               ("qwen3_moe", qwen3_moe_config(s), decode_weight_bytes(s, batch, False))):
+            if label not in only_models:
+                continue
+            r = run_model(cfg, batch, prompt_len, args.steps, args.warmup)
+            r["decode_weight_bytes"] = wb
+            r["decode_weight_roofline_frac"] = wb / (r["ms_per_decode_step"] * 1e-3) / HBM_BYTES_PER_S
+            entry[label] = r
+        if "zedirax" in entry and "gazutar" in entry:
+            entry["zedirax_vs_gazutar"] = {k: entry["zedirax"][k] / entry["gazutar"][k] for k in ("prefill_tok_s", "decode_tok_s")}
         out["sizes"][name] = entry
     print(json.dumps(out), flush=True)
     return out

@@ -577,6 +577,190 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
   }
 }
 
+// The matrix-core form for DECODE steps (one row per sequence) over a bf16 cache: a workgroup takes one (row, kv head) and
+// up to 16 of the query heads that read it - the heads are the 16 columns of the score tile where the prompt form has 16
+// consecutive rows of one head, so every K and V element the workgroup loads serves all of the group's heads (latent
+// attention: ONE cache row for every head).  Its four waves take the rounds of 32 keys in turn and merge their (max, sum,
+// accumulator) triples through LDS.  Arithmetic as in the prompt form: q and the softmax weights as bf16 hi + lo pairs.
+template <int DKM, int DVM, bool PAIR>
+__global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
+    const float* __restrict__ q, int64_t ldq, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_tables, int table_cols, const int32_t* __restrict__ kv_lens, int H, int G, int D,
+    int Dv, int block_size, int window, float scale, AttnBias bias, int64_t ldv, const float* __restrict__ gate,
+    int64_t ldg, float* __restrict__ out, int64_t ldo) {
+  __shared__ __attribute__((aligned(16))) float part_o[3][DVM][64][4];
+  __shared__ float part_ml[3][2][64];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int row = blockIdx.x, g = blockIdx.y;
+  const int hpg = H / G;
+  const int h0 = g * hpg + blockIdx.z * 16;               // first head of this workgroup's columns
+  const int nh = min(16, g * hpg + hpg - h0);             // valid columns
+  const int qi = lane & 15, kg = lane >> 4;
+  const int dk = D / 32, dvt = Dv / 16;
+  const int pos = kv_lens[row] - 1;
+  const int32_t* table = block_tables + (int64_t)row * table_cols;
+  const HeadBias hb = head_bias(bias, qi < nh ? h0 + qi : h0, H);
+  const bool q_vec = (ldq % 4 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15u) == 0) && (D % 4 == 0);
+  bf16x8 qh[DKM], ql[DKM];
+#pragma unroll
+  for (int ks = 0; ks < DKM; ++ks) {
+    float xv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (ks < dk && qi < nh) {
+      const float* qp = q + (int64_t)row * ldq + (int64_t)(h0 + qi) * D + ks * 32 + kg * 8;
+      if (q_vec) {
+        const float4 a = *reinterpret_cast<const float4*>(qp), b = *reinterpret_cast<const float4*>(qp + 4);
+        xv[0] = a.x, xv[1] = a.y, xv[2] = a.z, xv[3] = a.w, xv[4] = b.x, xv[5] = b.y, xv[6] = b.z, xv[7] = b.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[e] = qp[e];
+      }
+    }
+    float lo[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) lo[e] = xv[e] - rbf(xv[e]);
+    qh[ks] = as_frag(u32x4{pack_bf(xv[0], xv[1]), pack_bf(xv[2], xv[3]), pack_bf(xv[4], xv[5]), pack_bf(xv[6], xv[7])});
+    ql[ks] = as_frag(u32x4{pack_bf(lo[0], lo[1]), pack_bf(lo[2], lo[3]), pack_bf(lo[4], lo[5]), pack_bf(lo[6], lo[7])});
+  }
+  const int lo_key = max(0, pos - window + 1), hi_key = pos;
+  float m = -INFINITY, l = 0.f;
+  f32x4 oacc[DVM];
+#pragma unroll
+  for (int dt = 0; dt < DVM; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j0 = lo_key + 32 * wave; j0 <= hi_key; j0 += 32 * 4) {
+    f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int key = j0 + t * 16 + qi;  // (this lane's row of the K operand)
+      const bool ok = key <= hi_key;
+      const uint16_t* kr = k_cache;
+      if (ok) kr += (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
+#pragma unroll
+      for (int ks = 0; ks < DKM; ++ks) {
+        if (ks < dk) {
+          u32x4 kv = {0u, 0u, 0u, 0u};
+          if (ok) kv = *reinterpret_cast<const u32x4*>(kr + ks * 32);
+          const bf16x8 kf = as_frag(kv);
+          sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qh[ks], sacc[t], 0, 0, 0);
+          sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[ks], sacc[t], 0, 0, 0);
+        }
+      }
+    }
+    float sc[8];
+    bool vis[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
+      vis[e] = qi < nh && key <= hi_key;
+      sc[e] = vis[e] ? sacc[e >> 2][e & 3] * scale - dist_bias(hb, pos - key) : -INFINITY;
+      mx = fmaxf(mx, sc[e]);
+    }
+    mx = xor_max<32>(xor_max<16>(mx));
+    const float m_new = fmaxf(m, mx);
+    const float corr = m == -INFINITY ? 0.f : expf(m - m_new);
+    float pv[8], psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pv[e] = vis[e] ? expf(sc[e] - m_new) : 0.f;
+      psum += pv[e];
+    }
+    psum = xor_sum<32>(xor_sum<16>(psum));
+    l = l * corr + psum;
+    m = m_new;
+    float plo[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) plo[e] = pv[e] - rbf(pv[e]);
+    const bf16x8 ph = as_frag(u32x4{pack_bf(pv[0], pv[1]), pack_bf(pv[2], pv[3]), pack_bf(pv[4], pv[5]), pack_bf(pv[6], pv[7])});
+    const bf16x8 pl = as_frag(u32x4{pack_bf(plo[0], plo[1]), pack_bf(plo[2], plo[3]), pack_bf(plo[4], plo[5]), pack_bf(plo[6], plo[7])});
+    const uint16_t* vrow[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
+      vrow[e] = key <= hi_key
+                    ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
+                          (PAIR ? 2 * qi : qi)
+                    : nullptr;
+    }
+    if constexpr (PAIR) {
+#pragma unroll
+      for (int dp = 0; dp < DVM / 2; ++dp) {
+        if (2 * dp < dvt) {
+          uint32_t w[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e] = vrow[e] ? *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32) : 0u;
+          const bf16x8 v_even = as_frag(u32x4{(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16),
+                                              (w[4] & 0xffffu) | (w[5] << 16), (w[6] & 0xffffu) | (w[7] << 16)});
+          const bf16x8 v_odd = as_frag(u32x4{(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u),
+                                             (w[4] >> 16) | (w[5] & 0xffff0000u), (w[6] >> 16) | (w[7] & 0xffff0000u)});
+          oacc[2 * dp] *= corr;
+          oacc[2 * dp + 1] *= corr;
+          oacc[2 * dp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_even, ph, oacc[2 * dp], 0, 0, 0);
+          oacc[2 * dp] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_even, pl, oacc[2 * dp], 0, 0, 0);
+          oacc[2 * dp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_odd, ph, oacc[2 * dp + 1], 0, 0, 0);
+          oacc[2 * dp + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_odd, pl, oacc[2 * dp + 1], 0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < DVM; ++dt) {
+        if (dt < dvt) {
+          uint32_t ve[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ve[e] = vrow[e] ? (uint32_t)vrow[e][dt * 16] : 0u;
+          const bf16x8 vf = as_frag(u32x4{ve[0] | (ve[1] << 16), ve[2] | (ve[3] << 16), ve[4] | (ve[5] << 16), ve[6] | (ve[7] << 16)});
+          oacc[dt] *= corr;
+          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, oacc[dt], 0, 0, 0);
+          oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, oacc[dt], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // merge the four waves' partial results (same lane layout in every wave); a wave without a round has m = -inf, l = 0
+  if (wave > 0) {
+#pragma unroll
+    for (int dt = 0; dt < DVM; ++dt)
+      if (dt < dvt) *reinterpret_cast<f32x4*>(part_o[wave - 1][dt][lane]) = oacc[dt];
+    part_ml[wave - 1][0][lane] = m;
+    part_ml[wave - 1][1][lane] = l;
+  }
+  __syncthreads();
+  if (wave > 0 || qi >= nh) return;
+  float mm = m;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) mm = fmaxf(mm, part_ml[w][0][lane]);
+  const float f0 = m == -INFINITY ? 0.f : expf(m - mm);
+  l *= f0;
+#pragma unroll
+  for (int dt = 0; dt < DVM; ++dt) oacc[dt] *= f0;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const float mw = part_ml[w][0][lane];
+    const float f = mw == -INFINITY ? 0.f : expf(mw - mm);
+    l = fmaf(part_ml[w][1][lane], f, l);
+#pragma unroll
+    for (int dt = 0; dt < DVM; ++dt)
+      if (dt < dvt) {
+        const f32x4 o = *reinterpret_cast<const f32x4*>(part_o[w][dt][lane]);
+        oacc[dt] += o * f;
+      }
+  }
+  const float inv = 1.f / l;
+  const int64_t obase = (int64_t)row * ldo + (int64_t)(h0 + qi) * Dv;
+  const int64_t gbase = (int64_t)row * ldg + (int64_t)(h0 + qi) * Dv;
+#pragma unroll
+  for (int dt = 0; dt < DVM; ++dt) {
+    if (dt < dvt) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int d = PAIR ? (dt >> 1) * 32 + 2 * (kg * 4 + r) + (dt & 1) : dt * 16 + kg * 4 + r;
+        float o = oacc[dt][r] * inv;
+        if (gate) o *= sigmoid_f(gate[gbase + d]);
+        out[obase + d] = o;
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // short causal convolution with a carried tail
 // ---------------------------------------------------------------------------------------------------------------
@@ -1285,6 +1469,22 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
       else if (pair) MI_SWA_MFMA(8, 16, true);
       else MI_SWA_MFMA(8, 16, false);
 #undef MI_SWA_MFMA
+      return check_launch();
+    }
+  }
+  if constexpr (sizeof(TC) == 2) {
+    // decode steps (a row per sequence) over a bf16 cache: the matrix-core form with a kv head's query heads as columns
+    if (rows == n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0 && G <= 65535) {
+      const dim3 grid_h(rows, G, (H / G + 15) / 16);
+#define MI_HEADS_MFMA(DKM, DVM, PAIR)                                                                                  \
+  hipLaunchKernelGGL((paged_attention_heads_mfma_kernel<DKM, DVM, PAIR>), grid_h, dim3(256), 0, st, q, ldq, k, v, bt,   \
+                     cols, kv_lens, H, G, D, Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo)
+      const bool small = D <= 128 && Dv <= 128, pair = Dv % 32 == 0;
+      if (small && pair) MI_HEADS_MFMA(4, 8, true);
+      else if (small) MI_HEADS_MFMA(4, 8, false);
+      else if (pair) MI_HEADS_MFMA(8, 16, true);
+      else MI_HEADS_MFMA(8, 16, false);
+#undef MI_HEADS_MFMA
       return check_launch();
     }
   }

@@ -203,6 +203,48 @@ def test_log_biased_attention_on_the_matrix_cores(H, G, D, Dv, T, start, alias):
     assert (got - want).abs().max() <= 1e-4 * want.abs().max(), float((got - want).abs().max() / want.abs().max())
 
 
+@pytest.mark.parametrize("H,G,D,Dv,alias,window", [(4, 2, 64, 48, False, None), (8, 1, 128, 128, False, 70), (20, 1, 64, 48, True, None),
+                                                    (6, 6, 32, 16, False, None), (16, 1, 256, 192, True, None), (3, 1, 256, 224, True, 33)])
+def test_decode_attention_with_the_heads_as_columns(H, G, D, Dv, alias, window):
+    """Decode steps over a bf16 cache: a kv head's query heads are the columns of one matrix-core tile (more than 16 heads:
+    several tiles), four waves split the keys.  Sequences of 1 to 300 cached tokens (fewer keys than waves, a partial last
+    round), scattered pages, log-distance bias, with and without a window, values inside the key rows or apart."""
+    from nanovllm import _C, ops
+
+    g = torch.Generator().manual_seed(H * D + Dv)
+    bs, lens = 16, [1, 2, 31, 32, 33, 129, 300]
+    n_blocks = sum(-(-n // bs) for n in lens)
+    perm = torch.randperm(n_blocks + 2, generator=g)
+    kc = torch.zeros(n_blocks + 2, G, bs, D, dtype=torch.bfloat16)
+    vc = torch.zeros(n_blocks + 2, G, bs, Dv, dtype=torch.bfloat16)
+    tables = torch.full((len(lens), -(-max(lens) // bs)), -1, dtype=torch.int32)
+    r1, r2 = torch.rand(H, generator=g) + 0.2, torch.rand(H, generator=g) * 3
+    q = torch.randn(len(lens), H, D, generator=g)
+    want, used = [], 0
+    for i, n in enumerate(lens):
+        k = torch.randn(n, G, D, generator=g).bfloat16()
+        v = k[..., :Dv] if alias else torch.randn(n, G, Dv, generator=g).bfloat16()
+        nb = -(-n // bs)
+        tables[i, :nb] = perm[used:used + nb].to(torch.int32)
+        used += nb
+        for p in range(n):
+            kc[tables[i, p // bs], :, p % bs] = k[p]
+            vc[tables[i, p // bs], :, p % bs] = v[p]
+        dist = (n - 1 - torch.arange(n)).double()
+        s = torch.einsum("hd,jhd->hj", q[i].double(), k.double().repeat_interleave(H // G, 1)) * 0.11
+        s = s - r1.double().view(H, 1) * torch.log(1 + r2.double().view(H, 1) * dist)
+        if window is not None:
+            s = s.masked_fill(dist.view(1, n) >= window, float("-inf"))
+        want.append(torch.einsum("hj,jhd->hd", torch.softmax(s, -1), v.double().repeat_interleave(H // G, 1)))
+    want = torch.stack(want)
+    kc_d = kc.cuda()
+    got = ops.paged_attention_f32(q.reshape(len(lens), H * D).cuda(), kc_d, kc_d if alias else vc.cuda(), D if alias else Dv,
+                                  tables.cuda(), torch.arange(len(lens) + 1, dtype=torch.int32).cuda(),
+                                  torch.tensor(lens, dtype=torch.int32).cuda(), H, G, D, Dv, bs, window or 2 ** 31 - 1, 0.11,
+                                  _C.BIAS_LOG, r1.cuda(), r2.cuda()).cpu().double().view(len(lens), H, Dv)
+    assert (got - want).abs().max() <= 1e-4 * want.abs().max(), float((got - want).abs().max() / want.abs().max())
+
+
 # ------------------------------------------------------------------------------------------------ cuts of one sequence
 def test_whole_prompt(mixed_model, mixed_replay):
     cfg, w, _ = mixed_model
