@@ -739,12 +739,15 @@ int mi_gemm_any_batched(const float* x, int64_t ldx, int64_t x_batch, const void
 #define MI_BIAS_NONE  2
 /* mi_swa_attention with the bias named and the value rows ldv elements apart: v_cache may be k_cache itself with
  * ldv = D when a token's value is the first Dv channels of its key row (latent attention: G = 1).  window >= the longest
- * sequence: plain causal attention. */
+ * sequence: plain causal attention.  workspace (may be NULL; workspace_elems floats): lets decode steps with few
+ * (row, kv head) units spread each unit's keys over several workgroups - rows * H * 2 k * (2 + Dv) floats allow k of
+ * them, up to 16. */
 int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
                            int cache_dtype, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
                            const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv, int block_size,
                            int window, float scale, int bias_kind, const float* bias_p1, const float* bias_p2,
-                           const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream);
+                           const float* gate, int64_t ldg, float* out, int64_t ldo, float* workspace,
+                           int64_t workspace_elems, mi_stream stream);
 /* res += mult * y (y may be NULL); w != NULL: out = res / sqrt(mean(res^2) + eps) * (w + shift) per row. */
 int mi_add_rmsnorm_f32(float* res, int64_t ldr, const float* y, int64_t ldy, float mult, const float* w, float shift,
                        float eps, float* out, int64_t ldo, int rows, int width, mi_stream stream);

@@ -467,16 +467,15 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
       f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        const int key = j0 + t * 16 + qi;  // (this lane's row of the K operand)
-        const bool ok = key <= hi_key;
-        const uint16_t* kr = k_cache;
-        if (ok) kr += (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
+        // this lane's row of the K operand; rows beyond the last key repeat it (their scores are masked below), so
+        // that every load is unconditional and a round's loads are all in flight together
+        const int key = min(j0 + t * 16 + qi, hi_key);
+        const uint16_t* kr =
+            k_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
 #pragma unroll
         for (int ks = 0; ks < DKM; ++ks) {
           if (ks < dk) {
-            u32x4 kv = {0u, 0u, 0u, 0u};
-            if (ok) kv = *reinterpret_cast<const u32x4*>(kr + ks * 32);
-            const bf16x8 kf = as_frag(kv);
+            const bf16x8 kf = as_frag(*reinterpret_cast<const u32x4*>(kr + ks * 32));
             sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qh[ks], sacc[t], 0, 0, 0);
             sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[ks], sacc[t], 0, 0, 0);
           }
@@ -515,11 +514,9 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
       const uint16_t* vrow[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
-        vrow[e] = key <= hi_key
-                      ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
-                            (PAIR ? 2 * qi : qi)
-                      : nullptr;
+        const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
+        vrow[e] = v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
+                  (PAIR ? 2 * qi : qi);
       }
       if constexpr (PAIR) {
 #pragma unroll
@@ -527,7 +524,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
           if (2 * dp < dvt) {
             uint32_t w[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) w[e] = vrow[e] ? *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32) : 0u;
+            for (int e = 0; e < 8; ++e) w[e] = *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32);
             const bf16x8 v_even = as_frag(u32x4{(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16),
                                                 (w[4] & 0xffffu) | (w[5] << 16), (w[6] & 0xffffu) | (w[7] << 16)});
             const bf16x8 v_odd = as_frag(u32x4{(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u),
@@ -546,7 +543,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
           if (dt < dvt) {
             uint32_t ve[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) ve[e] = vrow[e] ? (uint32_t)vrow[e][dt * 16] : 0u;
+            for (int e = 0; e < 8; ++e) ve[e] = (uint32_t)vrow[e][dt * 16];
             const bf16x8 vf = as_frag(u32x4{ve[0] | (ve[1] << 16), ve[2] | (ve[3] << 16), ve[4] | (ve[5] << 16), ve[6] | (ve[7] << 16)});
             oacc[dt] *= corr;
             oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, oacc[dt], 0, 0, 0);
@@ -587,13 +584,14 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
     const float* __restrict__ q, int64_t ldq, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_tables, int table_cols, const int32_t* __restrict__ kv_lens, int H, int G, int D,
     int Dv, int block_size, int window, float scale, AttnBias bias, int64_t ldv, const float* __restrict__ gate,
-    int64_t ldg, float* __restrict__ out, int64_t ldo) {
+    int64_t ldg, float* __restrict__ out, int64_t ldo, int n_split, float* __restrict__ ws) {
   __shared__ __attribute__((aligned(16))) float part_o[3][DVM][64][4];
   __shared__ float part_ml[3][2][64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int row = blockIdx.x, g = blockIdx.y;
   const int hpg = H / G;
-  const int h0 = g * hpg + blockIdx.z * 16;               // first head of this workgroup's columns
+  const int split = blockIdx.z % n_split;                 // this workgroup's share of the rounds of keys
+  const int h0 = g * hpg + (blockIdx.z / n_split) * 16;   // first head of this workgroup's columns
   const int nh = min(16, g * hpg + hpg - h0);             // valid columns
   const int qi = lane & 15, kg = lane >> 4;
   const int dk = D / 32, dvt = Dv / 16;
@@ -626,20 +624,19 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
   f32x4 oacc[DVM];
 #pragma unroll
   for (int dt = 0; dt < DVM; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int j0 = lo_key + 32 * wave; j0 <= hi_key; j0 += 32 * 4) {
+  for (int j0 = lo_key + 32 * (split * 4 + wave); j0 <= hi_key; j0 += 32 * 4 * n_split) {
     f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int key = j0 + t * 16 + qi;  // (this lane's row of the K operand)
-      const bool ok = key <= hi_key;
-      const uint16_t* kr = k_cache;
-      if (ok) kr += (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
+      // this lane's row of the K operand; rows beyond the last key repeat it (their scores are masked below), so
+      // that every load is unconditional and a round's loads are all in flight together
+      const int key = min(j0 + t * 16 + qi, hi_key);
+      const uint16_t* kr =
+          k_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
 #pragma unroll
       for (int ks = 0; ks < DKM; ++ks) {
         if (ks < dk) {
-          u32x4 kv = {0u, 0u, 0u, 0u};
-          if (ok) kv = *reinterpret_cast<const u32x4*>(kr + ks * 32);
-          const bf16x8 kf = as_frag(kv);
+          const bf16x8 kf = as_frag(*reinterpret_cast<const u32x4*>(kr + ks * 32));
           sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qh[ks], sacc[t], 0, 0, 0);
           sacc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[ks], sacc[t], 0, 0, 0);
         }
@@ -675,11 +672,9 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
     const uint16_t* vrow[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
-      vrow[e] = key <= hi_key
-                    ? v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
-                          (PAIR ? 2 * qi : qi)
-                    : nullptr;
+      const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
+      vrow[e] = v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
+                (PAIR ? 2 * qi : qi);
     }
     if constexpr (PAIR) {
 #pragma unroll
@@ -687,7 +682,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
         if (2 * dp < dvt) {
           uint32_t w[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) w[e] = vrow[e] ? *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32) : 0u;
+          for (int e = 0; e < 8; ++e) w[e] = *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32);
           const bf16x8 v_even = as_frag(u32x4{(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16),
                                               (w[4] & 0xffffu) | (w[5] << 16), (w[6] & 0xffffu) | (w[7] << 16)});
           const bf16x8 v_odd = as_frag(u32x4{(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u),
@@ -706,7 +701,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
         if (dt < dvt) {
           uint32_t ve[8];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) ve[e] = vrow[e] ? (uint32_t)vrow[e][dt * 16] : 0u;
+          for (int e = 0; e < 8; ++e) ve[e] = (uint32_t)vrow[e][dt * 16];
           const bf16x8 vf = as_frag(u32x4{ve[0] | (ve[1] << 16), ve[2] | (ve[3] << 16), ve[4] | (ve[5] << 16), ve[6] | (ve[7] << 16)});
           oacc[dt] *= corr;
           oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, oacc[dt], 0, 0, 0);
@@ -744,6 +739,22 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
         oacc[dt] += o * f;
       }
   }
+  if (n_split > 1) {
+    // several workgroups share this (row, head): leave (max, sum, unnormalised accumulator) for the merge kernel
+    float* p = ws + (((int64_t)row * H + h0 + qi) * n_split + split) * (2 + Dv);
+    if (kg == 0) p[0] = mm, p[1] = l;
+#pragma unroll
+    for (int dt = 0; dt < DVM; ++dt) {
+      if (dt < dvt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int d = PAIR ? (dt >> 1) * 32 + 2 * (kg * 4 + r) + (dt & 1) : dt * 16 + kg * 4 + r;
+          p[2 + d] = oacc[dt][r];
+        }
+      }
+    }
+    return;
+  }
   const float inv = 1.f / l;
   const int64_t obase = (int64_t)row * ldo + (int64_t)(h0 + qi) * Dv;
   const int64_t gbase = (int64_t)row * ldg + (int64_t)(h0 + qi) * Dv;
@@ -758,6 +769,34 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
         out[obase + d] = o;
       }
     }
+  }
+}
+
+// the partial results of the workgroups that shared a (row, head) -> the output row; a wave per (row, head)
+__global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ ws, int n_split, int n_units,
+                                                                    int H, int Dv, const float* __restrict__ gate,
+                                                                    int64_t ldg, float* __restrict__ out, int64_t ldo) {
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (unit >= n_units) return;
+  const int row = unit / H, h = unit % H;
+  const float* p = ws + (int64_t)unit * n_split * (2 + Dv);
+  float mm = -INFINITY;
+  for (int sidx = 0; sidx < n_split; ++sidx) mm = fmaxf(mm, p[(int64_t)sidx * (2 + Dv)]);
+  float l = 0.f;
+  for (int sidx = 0; sidx < n_split; ++sidx) {
+    const float m = p[(int64_t)sidx * (2 + Dv)];
+    l = fmaf(p[(int64_t)sidx * (2 + Dv) + 1], m == -INFINITY ? 0.f : expf(m - mm), l);
+  }
+  const float inv = 1.f / l;
+  for (int d = lane; d < Dv; d += 64) {
+    float o = 0.f;
+    for (int sidx = 0; sidx < n_split; ++sidx) {
+      const float m = p[(int64_t)sidx * (2 + Dv)];
+      o = fmaf(p[(int64_t)sidx * (2 + Dv) + 2 + d], m == -INFINITY ? 0.f : expf(m - mm), o);
+    }
+    o *= inv;
+    if (gate) o *= sigmoid_f(gate[(int64_t)row * ldg + (int64_t)h * Dv + d]);
+    out[(int64_t)row * ldo + (int64_t)h * Dv + d] = o;
   }
 }
 
@@ -1452,7 +1491,7 @@ template <typename TC>
 static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* vc, const int32_t* bt, int cols,
                       const int32_t* cu_q, const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
                       int block_size, int window, float scale, AttnBias bias, int64_t ldv, const float* gate, int64_t ldg,
-                      float* out, int64_t ldo, hipStream_t st) {
+                      float* out, int64_t ldo, float* ws, int64_t ws_elems, hipStream_t st) {
   const TC* k = static_cast<const TC*>(kc);
   const TC* v = static_cast<const TC*>(vc);
   constexpr int VEC = 16 / sizeof(TC);
@@ -1475,16 +1514,28 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
   if constexpr (sizeof(TC) == 2) {
     // decode steps (a row per sequence) over a bf16 cache: the matrix-core form with a kv head's query heads as columns
     if (rows == n_seqs && D % 32 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 && ldv % 2 == 0 && G <= 65535) {
-      const dim3 grid_h(rows, G, (H / G + 15) / 16);
+      // few (row, kv head) units: up to 16 workgroups share one, each taking every n_split-th batch of four rounds, and
+      // a second launch merges their partial results (workspace: rows * H * n_split * (2 + Dv) floats)
+      const int chunks = (H / G + 15) / 16;
+      int n_split = 1;
+      while (n_split < 16 && (int64_t)rows * G * chunks * n_split < 512 &&
+             (int64_t)rows * H * (2 * n_split) * (2 + Dv) <= ws_elems)
+        n_split *= 2;
+      if (!ws) n_split = 1;
+      const dim3 grid_h(rows, G, chunks * n_split);
 #define MI_HEADS_MFMA(DKM, DVM, PAIR)                                                                                  \
   hipLaunchKernelGGL((paged_attention_heads_mfma_kernel<DKM, DVM, PAIR>), grid_h, dim3(256), 0, st, q, ldq, k, v, bt,   \
-                     cols, kv_lens, H, G, D, Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo)
+                     cols, kv_lens, H, G, D, Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo, n_split, ws)
       const bool small = D <= 128 && Dv <= 128, pair = Dv % 32 == 0;
       if (small && pair) MI_HEADS_MFMA(4, 8, true);
       else if (small) MI_HEADS_MFMA(4, 8, false);
       else if (pair) MI_HEADS_MFMA(8, 16, true);
       else MI_HEADS_MFMA(8, 16, false);
 #undef MI_HEADS_MFMA
+      if (check_launch() != MI_OK) return MI_ELAUNCH;
+      if (n_split == 1) return MI_OK;
+      hipLaunchKernelGGL(paged_attention_merge_kernel, dim3((rows * H + 3) / 4), dim3(256), 0, st, ws, n_split, rows * H, H,
+                         Dv, gate, ldg, out, ldo);
       return check_launch();
     }
   }
@@ -1526,7 +1577,7 @@ extern "C" int mi_swa_attention(const float* q, int64_t ldq, const void* k_cache
                                 float scale, const float* gate, int64_t ldg, float* out, int64_t ldo, mi_stream stream) {
   return mi_paged_attention_f32(q, ldq, k_cache, v_cache, Dv, cache_dtype, block_tables, table_cols, cu_q, kv_lens, n_seqs,
                                 rows, H, G, D, Dv, block_size, window, scale, MI_BIAS_SLOPE, nullptr, nullptr, gate, ldg,
-                                out, ldo, stream);
+                                out, ldo, nullptr, 0, stream);
 }
 
 extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, int64_t ldv,
@@ -1534,7 +1585,7 @@ extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k
                                       const int32_t* kv_lens, int n_seqs, int rows, int H, int G, int D, int Dv,
                                       int block_size, int window, float scale, int bias_kind, const float* bias_p1,
                                       const float* bias_p2, const float* gate, int64_t ldg, float* out, int64_t ldo,
-                                      mi_stream stream) {
+                                      float* workspace, int64_t workspace_elems, mi_stream stream) {
   if (!q || !k_cache || !v_cache || !block_tables || !cu_q || !kv_lens || !out || rows < 0 || n_seqs < 1) return MI_EINVAL;
   if (H < 1 || G < 1 || H % G || D < 1 || Dv < 1 || block_size < 1 || window < 1 || table_cols < 1 || ldv < Dv) return MI_EINVAL;
   if (bias_kind != MI_BIAS_SLOPE && bias_kind != MI_BIAS_LOG && bias_kind != MI_BIAS_NONE) return MI_EINVAL;
@@ -1544,10 +1595,12 @@ extern "C" int mi_paged_attention_f32(const float* q, int64_t ldq, const void* k
   const AttnBias bias{bias_kind, bias_p1, bias_p2};
   if (cache_dtype == MI_DTYPE_BF16)
     return launch_swa<uint16_t>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D,
-                                Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo, S(stream));
+                                Dv, block_size, window, scale, bias, ldv, gate, ldg, out, ldo, workspace, workspace_elems,
+                                S(stream));
   if (cache_dtype == MI_DTYPE_F32)
     return launch_swa<float>(q, ldq, k_cache, v_cache, block_tables, table_cols, cu_q, kv_lens, n_seqs, rows, H, G, D, Dv,
-                             block_size, window, scale, bias, ldv, gate, ldg, out, ldo, S(stream));
+                             block_size, window, scale, bias, ldv, gate, ldg, out, ldo, workspace, workspace_elems,
+                             S(stream));
   return MI_EINVAL;
 }
 

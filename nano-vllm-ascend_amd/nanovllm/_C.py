@@ -190,7 +190,7 @@ _SIGNATURES = {
     "mi_gemm_any_batched": (c_int, [_p, c_int64, c_int64, _p, c_int, _p, c_int64, c_int64, _p, c_int64, c_int64, c_int,
                                     c_int, c_int, c_int, c_int, _p]),
     "mi_paged_attention_f32": (c_int, [_p, c_int64, _p, _p, c_int64, c_int, _p, c_int, _p, _p, c_int, c_int, c_int, c_int,
-                                       c_int, c_int, c_int, c_int, c_float, c_int, _p, _p, _p, c_int64, _p, c_int64, _p]),
+                                       c_int, c_int, c_int, c_int, c_float, c_int, _p, _p, _p, c_int64, _p, c_int64, _p, c_int64, _p]),
     "mi_add_rmsnorm_f32": (c_int, [_p, c_int64, _p, c_int64, c_float, _p, c_float, c_float, _p, c_int64, c_int, c_int, _p]),
     "mi_depth_mix_f32": (c_int, [_p, c_int64, c_int, _p, _p, c_int64, c_float, _p, c_float, c_float, _p, c_int64, c_int,
                                  c_int, _p]),

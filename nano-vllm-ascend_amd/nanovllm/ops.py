@@ -1188,11 +1188,15 @@ def paged_attention_f32(q, k_cache, v_cache, ldv: int, block_tables, cu_q, kv_le
     assert k_cache.dtype == v_cache.dtype
     assert bias_kind != _C.BIAS_LOG or (bias_p1.numel() == H and bias_p2.numel() == H)
     out = torch.empty((rows, H * Dv), dtype=_F32, device=q.device)
+    ws = None
+    if rows == n_seqs and k_cache.dtype == _BF16:   # a decode step: room for up to 16 workgroups per (row, head)
+        ws = torch.empty(rows * H * 32 * (2 + Dv), dtype=_F32, device=q.device)
     check(lib.mi_paged_attention_f32(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), int(ldv), _dt(k_cache),
                                      ptr(block_tables), block_tables.shape[1], ptr(cu_q), ptr(kv_lens), n_seqs, rows, H, G,
                                      D, Dv, block_size, int(min(window, 2 ** 31 - 1)), float(scale), int(bias_kind),
                                      ptr(bias_p1), ptr(bias_p2), ptr(gate), gate.stride(0) if gate is not None else 0,
-                                     ptr(out), out.stride(0), stream()), "mi_paged_attention_f32")
+                                     ptr(out), out.stride(0), ptr(ws), ws.numel() if ws is not None else 0, stream()),
+          "mi_paged_attention_f32")
     return out
 
 
