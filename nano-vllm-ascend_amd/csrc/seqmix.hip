@@ -772,28 +772,36 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
   }
 }
 
-// the partial results of the workgroups that shared a (row, head) -> the output row; a wave per (row, head)
-__global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ ws, int n_split, int n_units,
-                                                                    int H, int Dv, const float* __restrict__ gate,
-                                                                    int64_t ldg, float* __restrict__ out, int64_t ldo) {
+// the partial results of the NS workgroups that shared a (row, head) -> the output row; a wave per (row, head), the
+// partials' loads unrolled (all in flight together)
+template <int NS>
+__global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ ws, int n_units, int H, int Dv,
+                                                                    const float* __restrict__ gate, int64_t ldg,
+                                                                    float* __restrict__ out, int64_t ldo) {
   const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (unit >= n_units) return;
   const int row = unit / H, h = unit % H;
-  const float* p = ws + (int64_t)unit * n_split * (2 + Dv);
-  float mm = -INFINITY;
-  for (int sidx = 0; sidx < n_split; ++sidx) mm = fmaxf(mm, p[(int64_t)sidx * (2 + Dv)]);
-  float l = 0.f;
-  for (int sidx = 0; sidx < n_split; ++sidx) {
-    const float m = p[(int64_t)sidx * (2 + Dv)];
-    l = fmaf(p[(int64_t)sidx * (2 + Dv) + 1], m == -INFINITY ? 0.f : expf(m - mm), l);
+  const int64_t stride = 2 + Dv;
+  const float* p = ws + (int64_t)unit * NS * stride;
+  float m[NS], f[NS];
+  float mm = -INFINITY, l = 0.f;
+#pragma unroll
+  for (int i = 0; i < NS; ++i) m[i] = p[i * stride];
+#pragma unroll
+  for (int i = 0; i < NS; ++i) mm = fmaxf(mm, m[i]);
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    f[i] = m[i] == -INFINITY ? 0.f : expf(m[i] - mm);
+    l = fmaf(p[i * stride + 1], f[i], l);
   }
   const float inv = 1.f / l;
   for (int d = lane; d < Dv; d += 64) {
+    float v[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) v[i] = p[i * stride + 2 + d];
     float o = 0.f;
-    for (int sidx = 0; sidx < n_split; ++sidx) {
-      const float m = p[(int64_t)sidx * (2 + Dv)];
-      o = fmaf(p[(int64_t)sidx * (2 + Dv) + 2 + d], m == -INFINITY ? 0.f : expf(m - mm), o);
-    }
+#pragma unroll
+    for (int i = 0; i < NS; ++i) o = fmaf(v[i], f[i], o);
     o *= inv;
     if (gate) o *= sigmoid_f(gate[(int64_t)row * ldg + (int64_t)h * Dv + d]);
     out[(int64_t)row * ldo + (int64_t)h * Dv + d] = o;
@@ -1534,8 +1542,14 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
 #undef MI_HEADS_MFMA
       if (check_launch() != MI_OK) return MI_ELAUNCH;
       if (n_split == 1) return MI_OK;
-      hipLaunchKernelGGL(paged_attention_merge_kernel, dim3((rows * H + 3) / 4), dim3(256), 0, st, ws, n_split, rows * H, H,
-                         Dv, gate, ldg, out, ldo);
+#define MI_MERGE(NS)                                                                                                  \
+  hipLaunchKernelGGL((paged_attention_merge_kernel<NS>), dim3((rows * H + 3) / 4), dim3(256), 0, st, ws, rows * H, H, Dv, \
+                     gate, ldg, out, ldo)
+      if (n_split == 2) MI_MERGE(2);
+      else if (n_split == 4) MI_MERGE(4);
+      else if (n_split == 8) MI_MERGE(8);
+      else MI_MERGE(16);
+#undef MI_MERGE
       return check_launch();
     }
   }
