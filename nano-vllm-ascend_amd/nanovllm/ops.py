@@ -1026,17 +1026,9 @@ def swa_prepare(proj, q_off: int, k_off: int, v_off: int, qn_w, kn_w, eps: float
 
 def swa_attention(q, k_cache, v_cache, block_tables, cu_q, kv_lens, H: int, G: int, D: int, Dv: int, block_size: int,
                   window: int, scale: float, gate=None) -> torch.Tensor:
-    require_gpu(q, k_cache, v_cache, block_tables, cu_q, kv_lens)
-    _f32(q, gate)
-    _i32(block_tables, cu_q, kv_lens)
-    rows, n_seqs = q.shape[0], kv_lens.numel()
-    assert q.shape[1] >= H * D and cu_q.numel() == n_seqs + 1 and block_tables.shape[0] >= n_seqs
-    out = torch.empty((rows, H * Dv), dtype=_F32, device=q.device)
-    check(lib.mi_swa_attention(ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), _dt(k_cache), ptr(block_tables),
-                               block_tables.shape[1], ptr(cu_q), ptr(kv_lens), n_seqs, rows, H, G, D, Dv, block_size,
-                               int(window), float(scale), ptr(gate), gate.stride(0) if gate is not None else 0,
-                               ptr(out), out.stride(0), stream()), "mi_swa_attention")
-    return out
+    """Paged sliding-window attention with the per-head geometric distance slopes (see paged_attention_f32)."""
+    return paged_attention_f32(q, k_cache, v_cache, Dv, block_tables, cu_q, kv_lens, H, G, D, Dv, block_size, window, scale,
+                               _C.BIAS_SLOPE, None, None, gate)
 
 
 def causal_conv_silu(x, w, state, cu_q, kv_lens, slot_ids) -> torch.Tensor:
