@@ -1246,12 +1246,23 @@ __global__ __launch_bounds__(256) void mingru_summary_kernel(const float* __rest
   const ScanSeg sg = scan_segment(cu_q, n_seqs, blockIdx.y);
   if (c >= width || sg.count == 0 || sg.index + 1 == sg.total) return;
   float A = 1.f, B = 0.f;
-  for (int r = 0; r < sg.count; ++r) {
-    const float* row = proj + (int64_t)(sg.first + r) * ld;
-    float keep, add;
-    mingru_gates(row[z_off + c], row[x_off + c], keep, add);
-    A *= keep;
-    B = fmaf(keep, B, add);
+  // eight rows' operands are fetched before the first of them is used: the loads do not depend on the running pair
+  for (int r0 = 0; r0 < sg.count; r0 += 8) {
+    float zp[8], up[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float* row = proj + (int64_t)(sg.first + min(r0 + i, sg.count - 1)) * ld;
+      zp[i] = row[z_off + c], up[i] = row[x_off + c];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (r0 + i < sg.count) {
+        float keep, add;
+        mingru_gates(zp[i], up[i], keep, add);
+        A *= keep;
+        B = fmaf(keep, B, add);
+      }
+    }
   }
   summary[((int64_t)blockIdx.y * 2) * width + c] = A;
   summary[((int64_t)blockIdx.y * 2 + 1) * width + c] = B;
@@ -1292,13 +1303,22 @@ __global__ __launch_bounds__(256) void mingru_walk_kernel(const float* __restric
   float S;
   if (CARRIED) S = summary[((int64_t)blockIdx.y * 2) * width + c];
   else S = kv_lens[sg.s] - (cu_q[sg.s + 1] - cu_q[sg.s]) > 0 ? state[(int64_t)slot_ids[sg.s] * width + c] : 0.f;
-  for (int r = 0; r < sg.count; ++r) {
-    const float* row = proj + (int64_t)(sg.first + r) * ld;
-    float keep, add;
-    mingru_gates(row[z_off + c], row[x_off + c], keep, add);
-    S = fmaf(keep, S, add);
-    const float g = row[g_off + c];
-    out[(int64_t)(sg.first + r) * ldo + c] = S * (g / (1.f + expf(-g)));
+  for (int r0 = 0; r0 < sg.count; r0 += 8) {
+    float zp[8], up[8], gp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float* row = proj + (int64_t)(sg.first + min(r0 + i, sg.count - 1)) * ld;
+      zp[i] = row[z_off + c], up[i] = row[x_off + c], gp[i] = row[g_off + c];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (r0 + i < sg.count) {
+        float keep, add;
+        mingru_gates(zp[i], up[i], keep, add);
+        S = fmaf(keep, S, add);
+        out[(int64_t)(sg.first + r0 + i) * ldo + c] = S * (gp[i] / (1.f + expf(-gp[i])));
+      }
+    }
   }
   if (sg.index + 1 == sg.total) state[(int64_t)slot_ids[sg.s] * width + c] = S;
 }
