@@ -48,7 +48,7 @@ def zedirax_config(s: dict) -> dict:
     dense = {"kind": "dense", "ff": 2 * W}
     order = [(rec, moe), (att, moe), (rec, dense), (lat, moe)]
     layers = [dict(order[i % 4][0], mlp=order[i % 4][1]) for i in range(s["layers"])]
-    return {"architecture": "Zedirax", "vocab": s["vocab"], "width": W, "residual_mult": 0.7, "norm": {"eps": 1e-6}, "layers": layers}
+    return {"architecture": "Zedirax", "vocab": s["vocab"], "width": W, "residual_mult": 0.5, "norm": {"eps": 1e-6}, "layers": layers}
 
 
 def zedirax_decode_weight_bytes(cfg: dict, batch: int) -> float:
