@@ -158,6 +158,18 @@ __device__ __forceinline__ float dist_bias(const HeadBias& hb, int dist) {
   return hb.log ? hb.a * log1pf(hb.b * (float)dist) : hb.a * (float)dist;
 }
 
+// Row of a token in a paged cache [blocks][kv heads][block_size][.]: (table[key / block_size] * G + g) * block_size +
+// key % block_size, in 32-bit arithmetic (rows of a cache are far fewer than 2^32; the byte offset is formed from it with
+// one 32 x 32 -> 64-bit multiply-add), the division a shift when block_size is a power of two (bs_shift >= 0).
+__device__ __forceinline__ int block_shift(int block_size) {
+  return (block_size & (block_size - 1)) == 0 ? __builtin_ctz((unsigned)block_size) : -1;
+}
+__device__ __forceinline__ uint32_t cache_row(const int32_t* table, int key, int G, int g, int block_size, int bs_shift) {
+  const int blk = bs_shift >= 0 ? key >> bs_shift : key / block_size;
+  const int off = bs_shift >= 0 ? key & (block_size - 1) : key - blk * block_size;
+  return ((uint32_t)table[blk] * (uint32_t)G + (uint32_t)g) * (uint32_t)block_size + (uint32_t)off;
+}
+
 // The general form (any head sizes): one wave per (row, head); lanes over keys for the scores, over value channels for
 // the output, element-wise loads.
 template <typename TC, int VPL>  // VPL: value channels per lane (Dv <= 64 * VPL)
@@ -430,6 +442,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
   const HeadBias hb = head_bias(bias, h, H);
   const int qi = lane & 15, kg = lane >> 4;
   const int dk = D / 32, dvt = Dv / 16;
+  const int bs_shift = block_shift(block_size);
   const bool q_vec = (ldq % 4 == 0) && ((reinterpret_cast<uintptr_t>(q) & 15u) == 0) && (D % 4 == 0);
   const int group_end = min(rg * 16 + 16, n_rows);
   for (int first = rg * 16; first < group_end;) {
@@ -471,7 +484,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
         // that every load is unconditional and a round's loads are all in flight together
         const int key = min(j0 + t * 16 + qi, hi_key);
         const uint16_t* kr =
-            k_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
+            k_cache + (int64_t)cache_row(table, key, G, g, block_size, bs_shift) * D + kg * 8;
 #pragma unroll
         for (int ks = 0; ks < DKM; ++ks) {
           if (ks < dk) {
@@ -483,12 +496,27 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
       }
       float sc[8];
       bool vis[8];
+      int dist[8];
       float mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
         vis[e] = qi < nr && key <= my_pos && key > my_pos - window;
-        sc[e] = vis[e] ? sacc[e >> 2][e & 3] * scale - dist_bias(hb, my_pos - key) : -INFINITY;
+        sc[e] = sacc[e >> 2][e & 3] * scale;
+        dist[e] = my_pos - key;
+      }
+      // the bias kind is the same for the whole launch: a branch every wave takes the same way, so that the logarithms
+      // are not evaluated (and thrown away) where the bias is linear or absent
+      if (bias.kind == MI_BIAS_LOG) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sc[e] -= hb.a * log1pf(hb.b * (float)max(dist[e], 0));
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sc[e] -= hb.a * (float)dist[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        sc[e] = vis[e] ? sc[e] : -INFINITY;
         mx = fmaxf(mx, sc[e]);
       }
       mx = xor_max<32>(xor_max<16>(mx));
@@ -515,7 +543,7 @@ __global__ __launch_bounds__(256) void swa_attention_mfma_kernel(const float* __
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
-        vrow[e] = v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
+        vrow[e] = v_cache + (int64_t)cache_row(table, key, G, g, block_size, bs_shift) * (int)ldv +
                   (PAIR ? 2 * qi : qi);
       }
       if constexpr (PAIR) {
@@ -595,6 +623,7 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
   const int nh = min(16, g * hpg + hpg - h0);             // valid columns
   const int qi = lane & 15, kg = lane >> 4;
   const int dk = D / 32, dvt = Dv / 16;
+  const int bs_shift = block_shift(block_size);
   const int pos = kv_lens[row] - 1;
   const int32_t* table = block_tables + (int64_t)row * table_cols;
   const HeadBias hb = head_bias(bias, qi < nh ? h0 + qi : h0, H);
@@ -626,13 +655,32 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
   for (int dt = 0; dt < DVM; ++dt) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int j0 = lo_key + 32 * (split * 4 + wave); j0 <= hi_key; j0 += 32 * 4 * n_split) {
     f32x4 sacc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    // the round's V words are requested together with its K rows (their addresses do not depend on the scores): one
+    // memory latency per round instead of two behind one another.  The V^T operand: the lane's eight keys (its
+    // contraction slots) at two neighbouring channels per 32-channel pair of tiles (PAIR), else one channel per tile
+    const uint16_t* vrow[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
+      vrow[e] = v_cache + (int64_t)cache_row(table, key, G, g, block_size, bs_shift) * (int)ldv +
+                (PAIR ? 2 * qi : qi);
+    }
+    uint32_t vw[PAIR ? DVM / 2 : 1][8];
+    if constexpr (PAIR) {
+#pragma unroll
+      for (int dp = 0; dp < DVM / 2; ++dp)
+        if (2 * dp < dvt) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) vw[dp][e] = *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32);
+        }
+    }
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       // this lane's row of the K operand; rows beyond the last key repeat it (their scores are masked below), so
       // that every load is unconditional and a round's loads are all in flight together
       const int key = min(j0 + t * 16 + qi, hi_key);
       const uint16_t* kr =
-          k_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * D + kg * 8;
+          k_cache + (int64_t)cache_row(table, key, G, g, block_size, bs_shift) * D + kg * 8;
 #pragma unroll
       for (int ks = 0; ks < DKM; ++ks) {
         if (ks < dk) {
@@ -644,12 +692,26 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
     }
     float sc[8];
     bool vis[8];
+    int dist[8];
     float mx = -INFINITY;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int key = j0 + (e >> 2) * 16 + kg * 4 + (e & 3);
       vis[e] = qi < nh && key <= hi_key;
-      sc[e] = vis[e] ? sacc[e >> 2][e & 3] * scale - dist_bias(hb, pos - key) : -INFINITY;
+      sc[e] = sacc[e >> 2][e & 3] * scale;
+      dist[e] = pos - key;
+    }
+    // (the bias kind is the same for the whole launch: see the prompt form)
+    if (bias.kind == MI_BIAS_LOG) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc[e] -= hb.a * log1pf(hb.b * (float)max(dist[e], 0));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc[e] -= hb.a * (float)dist[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sc[e] = vis[e] ? sc[e] : -INFINITY;
       mx = fmaxf(mx, sc[e]);
     }
     mx = xor_max<32>(xor_max<16>(mx));
@@ -669,20 +731,11 @@ __global__ __launch_bounds__(256) void paged_attention_heads_mfma_kernel(
     for (int e = 0; e < 8; ++e) plo[e] = pv[e] - rbf(pv[e]);
     const bf16x8 ph = as_frag(u32x4{pack_bf(pv[0], pv[1]), pack_bf(pv[2], pv[3]), pack_bf(pv[4], pv[5]), pack_bf(pv[6], pv[7])});
     const bf16x8 pl = as_frag(u32x4{pack_bf(plo[0], plo[1]), pack_bf(plo[2], plo[3]), pack_bf(plo[4], plo[5]), pack_bf(plo[6], plo[7])});
-    const uint16_t* vrow[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int key = min(j0 + (e >> 2) * 16 + kg * 4 + (e & 3), hi_key);  // (beyond the last key: weight 0)
-      vrow[e] = v_cache + (((int64_t)table[key / block_size] * G + g) * block_size + key % block_size) * ldv +
-                (PAIR ? 2 * qi : qi);
-    }
     if constexpr (PAIR) {
 #pragma unroll
       for (int dp = 0; dp < DVM / 2; ++dp) {
         if (2 * dp < dvt) {
-          uint32_t w[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) w[e] = *reinterpret_cast<const uint32_t*>(vrow[e] + dp * 32);
+          const uint32_t(&w)[8] = vw[dp];
           const bf16x8 v_even = as_frag(u32x4{(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16),
                                               (w[4] & 0xffffu) | (w[5] << 16), (w[6] & 0xffffu) | (w[7] << 16)});
           const bf16x8 v_odd = as_frag(u32x4{(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u),
@@ -1546,7 +1599,7 @@ static int launch_swa(const float* q, int64_t ldq, const void* kc, const void* v
       // a second launch merges their partial results (workspace: rows * H * n_split * (2 + Dv) floats)
       const int chunks = (H / G + 15) / 16;
       int n_split = 1;
-      while (n_split < 16 && (int64_t)rows * G * chunks * n_split < 512 &&
+      while (n_split < 16 && (int64_t)rows * G * chunks * n_split < 256 &&
              (int64_t)rows * H * (2 * n_split) * (2 + Dv) <= ws_elems)
         n_split *= 2;
       if (!ws) n_split = 1;
